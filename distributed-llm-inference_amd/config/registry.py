@@ -1,7 +1,7 @@
 """One registry from an architecture's name to its configuration class and model builder.
 
-``config.json["architectures"][0]`` chooses the entry (``model_type`` is the fallback for folders
-that omit it). An entry holds the typed configuration's parser and a function that turns a parsed
+``config.json["architectures"][0]`` (or a string under ``"architecture"``) chooses the entry
+(``model_type`` is the fallback for folders that omit both). An entry holds the typed configuration's parser and a function that turns a parsed
 configuration into a :class:`dli_amd.parts.spec.ModelSpec`: the list of parts that the model is put
 together from. Registering a new architecture touches no file of the framework::
 
@@ -56,7 +56,9 @@ def registered_architectures() -> tuple[str, ...]:
 
 def resolve_architecture(cfg: Mapping[str, Any]) -> Architecture:
     """Pick the registry entry that a ``config.json`` dictionary names."""
-    names = cfg.get("architectures") or []
+    names = list(cfg.get("architectures") or [])
+    if isinstance(cfg.get("architecture"), str):  # a configuration that names its one architecture in the singular
+        names.append(cfg["architecture"])
     for name in names:
         if name in _ARCHITECTURES:
             return _ARCHITECTURES[name]

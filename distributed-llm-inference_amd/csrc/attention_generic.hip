@@ -11,8 +11,31 @@
 // Scores are scaled by `scale` (1/sqrt(head_dim) in the reference: src/dli/model/llama.py:165-177,
 // src/dli/model/paged_attention.py:150,274).
 //
-// Page layout: K [pages][kv_heads][page_size][head_dim], V [pages][kv_heads][head_dim][page_size].
+//
+// Optional changes to the scores, each a parameter (all off: plain causal softmax attention):
+//   chunk > 0     a query also sees only keys of its own chunk, floor(j / chunk) == floor(p / chunk),
+//                 chunks counted from position 0 of the request;
+//   r1, r2        per query head, r1[h] * log(1 + r2[h] * (p - j)) is taken off the scaled score;
+//   sink != 0     the softmax's denominator has one more term, exp(0): a key of score 0 without a
+//                 value, so a row's weights may add up to less than one;
+//   value_dim     the size of a value where it differs from a key's;
+//   gate          float32 [tokens][gate_stride]: the result is multiplied by sigmoid(gate) element
+//                 by element (same layout as the output).
+// tile_entry == nullptr: tile t is the single row of entry t (steps of single tokens, whose
+// launches read nothing that the host made from the step's lengths).
+//
+// Page layout: K [pages][kv_heads][page_size][head_dim], V [pages][kv_heads][value_dim][page_size].
 #include "common.h"
+
+struct ScoreChanges {
+  int chunk;
+  int sink;
+  const float* r1;
+  const float* r2;
+  int value_dim;
+  const float* gate;
+  int64_t gate_stride;
+};
 
 template <typename T, int RM, int RN, int DC>
 __global__ __launch_bounds__(256) void attention_generic_kernel(
@@ -21,7 +44,7 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
     const int* __restrict__ q_start, const int* __restrict__ kv_len,
     const int* __restrict__ block_tables, int table_stride, const int* __restrict__ tile_entry,
     const int* __restrict__ tile_q0, int q_heads, int kv_heads, int head_dim, int page_size,
-    float scale, int window) {
+    float scale, int window, ScoreChanges sc) {
   constexpr int BM = 16 * RM, BN = 16 * RN, DMAX = 16 * DC;
   __shared__ float qs[BM][DMAX + 1];
   __shared__ float ks[BN][DMAX + 1];
@@ -29,9 +52,11 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
   __shared__ float ps[BM][BN + 1];
 
   const int tid = threadIdx.x, tx = tid % 16, ty = tid / 16;
-  const int entry = tile_entry[blockIdx.x];
-  const int q0 = tile_q0[blockIdx.x];
+  const int entry = tile_entry != nullptr ? tile_entry[blockIdx.x] : blockIdx.x;
+  const int q0 = tile_entry != nullptr ? tile_q0[blockIdx.x] : 0;
   const int head = blockIdx.y;
+  const int value_dim = sc.value_dim;
+  const float r1 = sc.r1 != nullptr ? sc.r1[head] : 0.f, r2 = sc.r1 != nullptr ? sc.r2[head] : 0.f;
   const int kvh = head / (q_heads / kv_heads);
   const int tok0 = q_start[entry];
   const int q_len = q_start[entry + 1] - tok0;
@@ -48,16 +73,18 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
   float m_run[RM], l_run[RM], acc[RM][DC];
 #pragma unroll
   for (int i = 0; i < RM; ++i) {
-    m_run[i] = -INFINITY;
-    l_run[i] = 0.f;
+    m_run[i] = sc.sink ? 0.f : -INFINITY;  // the sink: a key of score 0 that brings no value
+    l_run[i] = sc.sink ? 1.f : 0.f;
 #pragma unroll
     for (int c = 0; c < DC; ++c) acc[i][c] = 0.f;
   }
 
   const int pos_lo = first_pos + q0, pos_hi = first_pos + q0 + rows - 1;
   int j_begin = 0;
-  if (window > 0) j_begin = max(0, pos_lo - window + 1) / BN * BN;
-  const int j_end = pos_hi + 1;
+  if (window > 0) j_begin = max(0, pos_lo - window + 1);
+  if (sc.chunk > 0) j_begin = max(j_begin, pos_lo / sc.chunk * sc.chunk);
+  j_begin = j_begin / BN * BN;
+  const int j_end = rows > 0 ? pos_hi + 1 : 0;
 
   for (int j0 = j_begin; j0 < j_end; j0 += BN) {
     __syncthreads();  // previous tile's reads of ks/vs/ps are done (and qs is written)
@@ -71,13 +98,13 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
       }
       ks[r][c] = kv;
     }
-    for (int idx = tid; idx < BN * head_dim; idx += 256) {
+    for (int idx = tid; idx < BN * value_dim; idx += 256) {
       const int c = idx / BN, r = idx - c * BN;  // key index fastest: contiguous in a V page
       const int j = j0 + r;
       float vv = 0.f;
       if (j < j_end) {
         const int64_t page = table[j / page_size];
-        vv = to_f32(v_pages[((page * kv_heads + kvh) * head_dim + c) * page_size + j % page_size]);
+        vv = to_f32(v_pages[((page * kv_heads + kvh) * value_dim + c) * page_size + j % page_size]);
       }
       vs[r][c] = vv;
     }
@@ -108,7 +135,9 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
 #pragma unroll
       for (int jj = 0; jj < RN; ++jj) {
         const int j = j0 + tx + 16 * jj;
-        const bool visible = r < rows && j <= pos && (window <= 0 || j > pos - window);
+        const bool visible = r < rows && j <= pos && (window <= 0 || j > pos - window) &&
+                             (sc.chunk <= 0 || j / sc.chunk == pos / sc.chunk);
+        if (sc.r1 != nullptr && visible) s[i][jj] -= r1 * log1pf(r2 * (float)(pos - j));
         s[i][jj] = visible ? s[i][jj] : -INFINITY;
         tile_max = fmaxf(tile_max, s[i][jj]);
       }
@@ -143,7 +172,7 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
       for (int i = 0; i < RM; ++i) pv[i] = ps[ty * RM + i][jj];
 #pragma unroll
       for (int c = 0; c < DC; ++c) {
-        if (c * 16 < head_dim) {
+        if (c * 16 < value_dim) {
           const float vv = vs[jj][tx + 16 * c];
 #pragma unroll
           for (int i = 0; i < RM; ++i) acc[i][c] = fmaf(pv[i], vv, acc[i][c]);
@@ -157,10 +186,16 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
     const int r = ty * RM + i;
     if (r >= rows) continue;
     const float inv = l_run[i] > 0.f ? 1.f / l_run[i] : 0.f;
-    T* o = out + (int64_t)(tok0 + q0 + r) * out_stride + (int64_t)head * head_dim;
+    T* o = out + (int64_t)(tok0 + q0 + r) * out_stride + (int64_t)head * value_dim;
+    const float* g = sc.gate != nullptr ? sc.gate + (int64_t)(tok0 + q0 + r) * sc.gate_stride + (int64_t)head * value_dim
+                                        : nullptr;
 #pragma unroll
     for (int c = 0; c < DC; ++c)
-      if (c * 16 < head_dim) o[tx + 16 * c] = from_f32<T>(acc[i][c] * inv);
+      if (tx + 16 * c < value_dim) {
+        float y = acc[i][c] * inv;
+        if (g != nullptr) y *= 1.f / (1.f + expf(-g[tx + 16 * c]));
+        o[tx + 16 * c] = from_f32<T>(y);
+      }
   }
 }
 
@@ -169,18 +204,51 @@ static int launch_generic(const void* q, int64_t q_stride, const void* k_pages, 
                           void* out, int64_t out_stride, const int* q_start, const int* kv_len,
                           const int* block_tables, int table_stride, const int* tile_entry,
                           const int* tile_q0, int tiles, int q_heads, int kv_heads, int head_dim,
-                          int page_size, float scale, int window, hipStream_t stream) {
+                          int page_size, float scale, int window, ScoreChanges sc, hipStream_t stream) {
   attention_generic_kernel<T, RM, RN, DC><<<dim3(tiles, q_heads), 256, 0, stream>>>(
       (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, q_start,
       kv_len, block_tables, table_stride, tile_entry, tile_q0, q_heads, kv_heads, head_dim,
-      page_size, scale, window);
+      page_size, scale, window, sc);
   return dli_launch_status();
 }
 
-// Queries per tile for a head_dim: the host builds its tile list with this.
+// Queries per tile for a head_dim (the larger of the key's and the value's size): the host builds
+// its tile list with this.
 extern "C" int dli_attention_generic_tile_rows(int head_dim) {
-  if (head_dim <= 0 || head_dim % 16 != 0 || head_dim > 256) return DLI_ERR_ARGUMENT;
+  if (head_dim <= 0 || head_dim > 256) return DLI_ERR_ARGUMENT;
   return head_dim <= 128 ? 32 : 16;
+}
+
+// The attention with every change to the scores as a parameter (see the head of this file).
+// chunk 0, sink 0, r1 = r2 = gate = nullptr and value_dim == head_dim: the plain attention.
+extern "C" int dli_attention_scored(const void* q, int64_t q_stride, const void* k_pages,
+                                    const void* v_pages, void* out, int64_t out_stride,
+                                    const int* q_start, const int* kv_len, const int* block_tables,
+                                    int table_stride, const int* tile_entry, const int* tile_q0,
+                                    int tiles, int q_heads, int kv_heads, int head_dim, int value_dim,
+                                    int page_size, float scale, int window, int chunk, int sink,
+                                    const float* r1, const float* r2, const float* gate,
+                                    int64_t gate_stride, int is_bf16, hipStream_t stream) {
+  if (tiles <= 0) return DLI_OK;
+  const int dmax = head_dim > value_dim ? head_dim : value_dim;
+  if (head_dim <= 0 || value_dim <= 0 || dmax > 256 || q_heads <= 0 || kv_heads <= 0 ||
+      q_heads % kv_heads != 0 || q_heads > 65535 || page_size <= 0 || table_stride <= 0 ||
+      window < 0 || chunk < 0 || (r1 == nullptr) != (r2 == nullptr) ||
+      (tile_entry == nullptr) != (tile_q0 == nullptr))
+    return DLI_ERR_ARGUMENT;
+  const ScoreChanges sc = {chunk, sink, r1, r2, value_dim, gate, gate_stride};
+#define GENERIC_ARGS                                                                              \
+  q, q_stride, k_pages, v_pages, out, out_stride, q_start, kv_len, block_tables, table_stride,   \
+      tile_entry, tile_q0, tiles, q_heads, kv_heads, head_dim, page_size, scale, window, sc, stream
+  if (is_bf16) {
+    if (dmax <= 64) return launch_generic<bf16_t, 2, 2, 4>(GENERIC_ARGS);
+    if (dmax <= 128) return launch_generic<bf16_t, 2, 2, 8>(GENERIC_ARGS);
+    return launch_generic<bf16_t, 1, 1, 16>(GENERIC_ARGS);
+  }
+  if (dmax <= 64) return launch_generic<float, 2, 2, 4>(GENERIC_ARGS);
+  if (dmax <= 128) return launch_generic<float, 2, 2, 8>(GENERIC_ARGS);
+  return launch_generic<float, 1, 1, 16>(GENERIC_ARGS);
+#undef GENERIC_ARGS
 }
 
 extern "C" int dli_attention_generic(const void* q, int64_t q_stride, const void* k_pages,
@@ -189,20 +257,9 @@ extern "C" int dli_attention_generic(const void* q, int64_t q_stride, const void
                                      int table_stride, const int* tile_entry, const int* tile_q0,
                                      int tiles, int q_heads, int kv_heads, int head_dim, int page_size,
                                      float scale, int window, int is_bf16, hipStream_t stream) {
-  if (tiles <= 0) return DLI_OK;
-  if (head_dim <= 0 || head_dim % 16 != 0 || head_dim > 256 || q_heads <= 0 || kv_heads <= 0 ||
-      q_heads % kv_heads != 0 || q_heads > 65535 || page_size <= 0 || table_stride <= 0)
-    return DLI_ERR_ARGUMENT;
-#define GENERIC_ARGS                                                                              \
-  q, q_stride, k_pages, v_pages, out, out_stride, q_start, kv_len, block_tables, table_stride,   \
-      tile_entry, tile_q0, tiles, q_heads, kv_heads, head_dim, page_size, scale, window, stream
-  if (is_bf16) {
-    if (head_dim <= 64) return launch_generic<bf16_t, 2, 2, 4>(GENERIC_ARGS);
-    if (head_dim <= 128) return launch_generic<bf16_t, 2, 2, 8>(GENERIC_ARGS);
-    return launch_generic<bf16_t, 1, 1, 16>(GENERIC_ARGS);
-  }
-  if (head_dim <= 64) return launch_generic<float, 2, 2, 4>(GENERIC_ARGS);
-  if (head_dim <= 128) return launch_generic<float, 2, 2, 8>(GENERIC_ARGS);
-  return launch_generic<float, 1, 1, 16>(GENERIC_ARGS);
-#undef GENERIC_ARGS
+  if (head_dim % 16 != 0 || tile_entry == nullptr) return tiles <= 0 ? DLI_OK : DLI_ERR_ARGUMENT;
+  return dli_attention_scored(q, q_stride, k_pages, v_pages, out, out_stride, q_start, kv_len,
+                              block_tables, table_stride, tile_entry, tile_q0, tiles, q_heads,
+                              kv_heads, head_dim, head_dim, page_size, scale, window, 0, 0, nullptr,
+                              nullptr, nullptr, 0, is_bf16, stream);
 }

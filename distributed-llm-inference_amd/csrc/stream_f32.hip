@@ -1,0 +1,267 @@
+// Kernels for models whose residual stream is kept in 32-bit whatever the type of the matrix
+// products: the stream `x` is float32 [tokens][width]; T is the type of what the products read and
+// write (float on the 32-bit path, bf16 when serving). Statistics, sums, angles and activations
+// are 32-bit.
+//
+//   embed_sinusoid     x = table[id] + pe(position), pe[2i] = sin(p f_i), pe[2i+1] = cos(p f_i)
+//   cast_from_f32      the stream rounded to T, as the operand of a product
+//   norm_into_stream   x += w * y / sqrt(mean(y^2) + eps)   (a norm on a sublayer's output)
+//   rms_norm_from_f32  out(T) = w * x / sqrt(mean(x^2) + eps)
+//   softcap            y = cap * tanh(y / cap)
+//   token_shift        S mixes of each row with the row before it, x + (prev - x) * mu_s; the row
+//                      before a step's first row comes from the request's state, which then
+//                      receives the step's last row
+//   lowrank_out        y = bias + W2 act(t): the second half of a low-rank projection, 32-bit
+//   qk_unit_cache      per-head unit RMS of q and k, value mixing, cache write
+#include "common.h"
+
+template <typename T>
+__global__ void embed_sinusoid_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                                      const int* __restrict__ positions, const float* __restrict__ inv_freq,
+                                      float* __restrict__ out, int width) {
+  const int64_t row = blockIdx.x;
+  const T* src = table + (int64_t)ids[row] * width;
+  const float p = (float)positions[row];
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float angle = p * inv_freq[i >> 1];
+    out[row * width + i] = to_f32(src[i]) + ((i & 1) ? cosf(angle) : sinf(angle));
+  }
+}
+
+template <typename T>
+__global__ void cast_from_f32_kernel(const float* __restrict__ x, T* __restrict__ out, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = from_f32<T>(x[i]);
+}
+
+template <typename T>
+__global__ void norm_into_stream_kernel(const T* __restrict__ y, int64_t y_stride, const float* __restrict__ weight,
+                                        float* __restrict__ x, int width, float eps) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  const T* yr = y + row * y_stride;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float f = to_f32(yr[i]);
+    ss += f * f;
+  }
+  const float r = 1.f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+  float* xr = x + row * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) xr[i] += weight[i] * (to_f32(yr[i]) * r);
+}
+
+template <typename T>
+__global__ void rms_norm_from_f32_kernel(const float* __restrict__ x, const float* __restrict__ weight,
+                                         T* __restrict__ out, int width, float eps) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  const float* xr = x + row * width;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) ss += xr[i] * xr[i];
+  const float r = 1.f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += blockDim.x) out[row * width + i] = from_f32<T>(weight[i] * (xr[i] * r));
+}
+
+__global__ void softcap_kernel(float* __restrict__ y, int64_t n, float cap) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) y[i] = cap * tanhf(y[i] / cap);
+}
+
+// The entry that holds `row`: the last e with q_start[e] <= row.
+__device__ __forceinline__ int entry_of_row(const int* __restrict__ q_start, int entries, int row) {
+  int lo = 0, hi = entries - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (q_start[mid] <= row) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
+// One workgroup a row. The thread that reads a request's state for the entry's first row is also
+// the one that writes the entry's last row there, after its read: no other thread touches that
+// element in this launch.
+template <typename T>
+__global__ void token_shift_kernel(const float* __restrict__ x, const float* __restrict__ mu, int mixes,
+                                   float* state, int64_t state_stride, const int* __restrict__ q_start, int entries,
+                                   const int* __restrict__ positions, const int* __restrict__ state_slots,
+                                   T* __restrict__ out, int rows, int width) {
+  const int row = blockIdx.x;
+  const int e = entry_of_row(q_start, entries, row);
+  const int first = q_start[e], last = q_start[e + 1] - 1;
+  const float* xr = x + (int64_t)row * width;
+  float* st = state + (int64_t)state_slots[e] * state_stride;
+  const bool from_state = row == first;
+  const bool fresh = positions[row] == 0;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float cur = xr[i];
+    float prev;
+    if (from_state) {
+      prev = fresh ? 0.f : st[i];
+      st[i] = x[(int64_t)last * width + i];
+    } else {
+      prev = xr[i - width];
+    }
+    for (int s = 0; s < mixes; ++s)
+      out[((int64_t)s * rows + row) * width + i] = from_f32<T>(cur + (prev - cur) * mu[(int64_t)s * width + i]);
+  }
+}
+
+// act: 0 none, 1 tanh. t is [rows][t_stride] (rank values a row), w2 [features][rank], out [rows][features].
+__global__ void lowrank_out_kernel(const float* __restrict__ t, int64_t t_stride, const float* __restrict__ w2,
+                                   const float* __restrict__ bias, float* __restrict__ out, int features, int rank,
+                                   int act) {
+  extern __shared__ float ts[];
+  const int64_t row = blockIdx.x;
+  for (int j = threadIdx.x; j < rank; j += blockDim.x) {
+    const float v = t[row * t_stride + j];
+    ts[j] = act == 1 ? tanhf(v) : v;
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < features; c += blockDim.x) {
+    float s = 0.f;
+    for (int j = 0; j < rank; ++j) s = fmaf(ts[j], w2[(int64_t)c * rank + j], s);
+    out[row * features + c] = s + (bias != nullptr ? bias[c] : 0.f);
+  }
+}
+
+// proj [tokens][stride] float32 holds q (q_heads x dim), k (kv_heads x dim) and v (kv_heads x vdim)
+// at the given column offsets. q and k are divided by their root mean square over dim, head by
+// head. v is mixed with the values that an earlier layer computed for the same token,
+// v <- (1 - lambda) v + lambda v_first (lambda == nullptr: no mixing; v_first_out != nullptr: this
+// layer's v is written there for the later ones). The unit k and the v that results go to the
+// token's cache slot (negative: not cached).
+template <typename T>
+__global__ void qk_unit_cache_kernel(const float* __restrict__ proj, int64_t stride, int q_off, int k_off, int v_off,
+                                     T* __restrict__ q_out, const float* __restrict__ lambda,
+                                     const float* __restrict__ v_first_in, float* __restrict__ v_first_out,
+                                     const int* __restrict__ slots, T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                     int q_heads, int kv_heads, int dim, int vdim, int page_size, float eps) {
+  const int64_t row = blockIdx.x;
+  const int lane = threadIdx.x % DLI_WAVE, wave = threadIdx.x / DLI_WAVE, waves = blockDim.x / DLI_WAVE;
+  const float* pr = proj + row * stride;
+  const int slot = slots[row];
+  const int64_t page = slot >= 0 ? slot / page_size : 0;
+  const int off = slot >= 0 ? slot % page_size : 0;
+  for (int h = wave; h < q_heads + kv_heads; h += waves) {
+    const bool is_q = h < q_heads;
+    const float* src = is_q ? pr + q_off + (int64_t)h * dim : pr + k_off + (int64_t)(h - q_heads) * dim;
+    float ss = 0.f;
+    for (int c = lane; c < dim; c += DLI_WAVE) ss += src[c] * src[c];
+    const float r = 1.f / sqrtf(wave_sum(ss) / (float)dim + eps);
+    if (is_q) {
+      for (int c = lane; c < dim; c += DLI_WAVE) q_out[(row * q_heads + h) * dim + c] = from_f32<T>(src[c] * r);
+    } else if (slot >= 0) {
+      T* dst = k_pages + ((page * kv_heads + (h - q_heads)) * page_size + off) * dim;
+      for (int c = lane; c < dim; c += DLI_WAVE) dst[c] = from_f32<T>(src[c] * r);
+    }
+  }
+  const float lam = lambda != nullptr ? lambda[0] : 0.f;
+  for (int i = threadIdx.x; i < kv_heads * vdim; i += blockDim.x) {
+    float v = pr[v_off + i];
+    if (lambda != nullptr) v = (1.f - lam) * v + lam * v_first_in[row * kv_heads * vdim + i];
+    if (v_first_out != nullptr) v_first_out[row * kv_heads * vdim + i] = v;
+    if (slot >= 0) {
+      const int g = i / vdim, c = i - g * vdim;
+      v_pages[((page * kv_heads + g) * vdim + c) * page_size + off] = from_f32<T>(v);
+    }
+  }
+}
+
+extern "C" {
+
+int dli_embed_sinusoid(const void* table, const int* ids, const int* positions, const float* inv_freq, float* out,
+                       int rows, int width, int is_bf16, hipStream_t stream) {
+  if (rows <= 0) return DLI_OK;
+  if (width <= 0) return DLI_ERR_ARGUMENT;
+  const int threads = width >= 1024 ? 256 : 128;
+  if (is_bf16)
+    embed_sinusoid_kernel<bf16_t><<<rows, threads, 0, stream>>>((const bf16_t*)table, ids, positions, inv_freq, out, width);
+  else
+    embed_sinusoid_kernel<float><<<rows, threads, 0, stream>>>((const float*)table, ids, positions, inv_freq, out, width);
+  return dli_launch_status();
+}
+
+int dli_cast_from_f32(const float* x, void* out, int64_t n, int is_bf16, hipStream_t stream) {
+  if (n <= 0) return DLI_OK;
+  const int64_t blocks = (n + 255) / 256;
+  if (blocks > 2147483647LL) return DLI_ERR_ARGUMENT;
+  if (is_bf16) cast_from_f32_kernel<bf16_t><<<(unsigned)blocks, 256, 0, stream>>>(x, (bf16_t*)out, n);
+  else cast_from_f32_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>(x, (float*)out, n);
+  return dli_launch_status();
+}
+
+int dli_norm_into_stream(const void* y, int64_t y_stride, const float* weight, float* x, int rows, int width, float eps,
+                         int y_is_bf16, hipStream_t stream) {
+  if (rows <= 0) return DLI_OK;
+  if (width <= 0 || y_stride < width) return DLI_ERR_ARGUMENT;
+  const int threads = width >= 2048 ? 512 : 256;
+  if (y_is_bf16)
+    norm_into_stream_kernel<bf16_t><<<rows, threads, 0, stream>>>((const bf16_t*)y, y_stride, weight, x, width, eps);
+  else
+    norm_into_stream_kernel<float><<<rows, threads, 0, stream>>>((const float*)y, y_stride, weight, x, width, eps);
+  return dli_launch_status();
+}
+
+int dli_rms_norm_from_f32(const float* x, const float* weight, void* out, int rows, int width, float eps, int is_bf16,
+                          hipStream_t stream) {
+  if (rows <= 0) return DLI_OK;
+  if (width <= 0) return DLI_ERR_ARGUMENT;
+  const int threads = width >= 2048 ? 512 : 256;
+  if (is_bf16)
+    rms_norm_from_f32_kernel<bf16_t><<<rows, threads, 0, stream>>>(x, weight, (bf16_t*)out, width, eps);
+  else
+    rms_norm_from_f32_kernel<float><<<rows, threads, 0, stream>>>(x, weight, (float*)out, width, eps);
+  return dli_launch_status();
+}
+
+int dli_softcap(float* y, int64_t n, float cap, hipStream_t stream) {
+  if (n <= 0) return DLI_OK;
+  const int64_t blocks = (n + 255) / 256;
+  if (!(cap > 0.f) || blocks > 2147483647LL) return DLI_ERR_ARGUMENT;
+  softcap_kernel<<<(unsigned)blocks, 256, 0, stream>>>(y, n, cap);
+  return dli_launch_status();
+}
+
+int dli_token_shift(const float* x, const float* mu, int mixes, float* state, int64_t state_stride, const int* q_start,
+                    int entries, const int* positions, const int* state_slots, void* out, int rows, int width,
+                    int is_bf16, hipStream_t stream) {
+  if (rows <= 0) return DLI_OK;
+  if (width <= 0 || mixes <= 0 || entries <= 0 || state_stride < width) return DLI_ERR_ARGUMENT;
+  const int threads = width >= 1024 ? 256 : 128;
+  if (is_bf16)
+    token_shift_kernel<bf16_t><<<rows, threads, 0, stream>>>(x, mu, mixes, state, state_stride, q_start, entries,
+                                                             positions, state_slots, (bf16_t*)out, rows, width);
+  else
+    token_shift_kernel<float><<<rows, threads, 0, stream>>>(x, mu, mixes, state, state_stride, q_start, entries,
+                                                            positions, state_slots, (float*)out, rows, width);
+  return dli_launch_status();
+}
+
+int dli_lowrank_out(const float* t, int64_t t_stride, const float* w2, const float* bias, float* out, int rows,
+                    int features, int rank, int act, hipStream_t stream) {
+  if (rows <= 0) return DLI_OK;
+  if (features <= 0 || rank <= 0 || rank > 8192 || t_stride < rank || act < 0 || act > 1) return DLI_ERR_ARGUMENT;
+  lowrank_out_kernel<<<rows, 256, rank * sizeof(float), stream>>>(t, t_stride, w2, bias, out, features, rank, act);
+  return dli_launch_status();
+}
+
+int dli_qk_unit_cache(const float* proj, int64_t stride, int q_off, int k_off, int v_off, void* q_out,
+                      const float* lambda, const float* v_first_in, float* v_first_out, const int* slots,
+                      void* k_pages, void* v_pages, int rows, int q_heads, int kv_heads, int dim, int vdim,
+                      int page_size, float eps, int is_bf16, hipStream_t stream) {
+  if (rows <= 0) return DLI_OK;
+  if (q_heads <= 0 || kv_heads <= 0 || dim <= 0 || vdim <= 0 || page_size <= 0 ||
+      (lambda != nullptr && v_first_in == nullptr))
+    return DLI_ERR_ARGUMENT;
+  if (is_bf16)
+    qk_unit_cache_kernel<bf16_t><<<rows, 256, 0, stream>>>(proj, stride, q_off, k_off, v_off, (bf16_t*)q_out, lambda,
+                                                           v_first_in, v_first_out, slots, (bf16_t*)k_pages,
+                                                           (bf16_t*)v_pages, q_heads, kv_heads, dim, vdim, page_size, eps);
+  else
+    qk_unit_cache_kernel<float><<<rows, 256, 0, stream>>>(proj, stride, q_off, k_off, v_off, (float*)q_out, lambda,
+                                                          v_first_in, v_first_out, slots, (float*)k_pages,
+                                                          (float*)v_pages, q_heads, kv_heads, dim, vdim, page_size, eps);
+  return dli_launch_status();
+}
+
+}  // extern "C"

@@ -97,6 +97,23 @@ _SIGNATURES = {
     "dli_attention_generic": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr,
                               _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
                               _c_int, _c_int, _c_ptr],
+    "dli_attention_scored": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr,
+                             _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_ptr,
+                             _c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr],
+    "dli_embed_sinusoid": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_cast_from_f32": [_c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr],
+    "dli_norm_into_stream": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+    "dli_rms_norm_from_f32": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+    "dli_softcap": [_c_ptr, _c_i64, _c_float, _c_ptr],
+    "dli_token_shift": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
+                        _c_int, _c_ptr],
+    "dli_lowrank_out": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_qk_unit_cache": [_c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+    "dli_recurrent_scan_supports": [_c_int],
+    "dli_recurrent_scan": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr,
+                           _c_i64, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64,
+                           _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
 }
 
 _lib: Optional[ctypes.CDLL] = None
@@ -1309,3 +1326,240 @@ def decode_advance(sampled: torch.Tensor, tokens_out: torch.Tensor, token_ids: t
         _ptr(sampled), _ptr(tokens_out), _ptr(token_ids), _ptr(positions), _ptr(kv_len), _ptr(counters),
         ctypes.cast(slot_ptrs, ctypes.c_void_p), ctypes.cast(table_ptrs, ctypes.c_void_p), n, width,
         int(page_size), rows, int(bool(advance)), _stream()), "decode_advance")
+
+
+# ----------------------------------------------------------------------------- a 32-bit residual stream
+
+def _f32_rows(t: torch.Tensor, name: str) -> None:
+    _rows(t, name, torch.float32)
+
+
+def embed_sinusoid(table: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor,
+                   out: torch.Tensor) -> None:
+    """``out[t] = table[ids[t]] + pe(positions[t])`` in float32, ``pe[2i] = sin(p f_i)``,
+    ``pe[2i+1] = cos(p f_i)`` with ``f = inv_freq [ceil(width/2)]``."""
+    _dense(table, "table", ndim=2)
+    _dense(ids, "ids", torch.int32, 1)
+    _dense(positions, "positions", torch.int32, 1)
+    _dense(inv_freq, "inv_freq", torch.float32, 1)
+    _dense(out, "out", torch.float32, 2)
+    n, width = ids.shape[0], table.shape[1]
+    _require(positions.shape[0] == n and out.shape == (n, width), "ids, positions and out disagree on the rows")
+    _require(inv_freq.shape[0] * 2 >= width, "inv_freq must hold a frequency for every pair of columns")
+    _check(library().dli_embed_sinusoid(_ptr(table), _ptr(ids), _ptr(positions), _ptr(inv_freq), _ptr(out), n, width,
+                                        _is_bf16(table.dtype), _stream()), "embed_sinusoid")
+
+
+def cast_from_f32(x: torch.Tensor, out: torch.Tensor) -> None:
+    """``out = x`` rounded to ``out``'s type (float32 or bfloat16)."""
+    _dense(x, "x", torch.float32)
+    _dense(out, "out")
+    _require(out.numel() == x.numel(), "out differs from x in size")
+    _check(library().dli_cast_from_f32(_ptr(x), _ptr(out), x.numel(), _is_bf16(out.dtype), _stream()), "cast_from_f32")
+
+
+def norm_into_stream(y: torch.Tensor, weight: torch.Tensor, eps: float, x: torch.Tensor) -> None:
+    """``x += weight * y / sqrt(mean(y^2) + eps)`` row by row: ``x`` float32 ``[n, width]``, ``y`` float32
+    or bfloat16 with contiguous rows, statistics and sum in 32-bit."""
+    _rows(y, "y", y.dtype)
+    _dense(x, "x", torch.float32, 2)
+    _dense(weight, "weight", torch.float32, 1)
+    _require(y.shape == x.shape and weight.shape[0] == x.shape[1], "y, x and weight disagree on the sizes")
+    _check(library().dli_norm_into_stream(_ptr(y), y.stride(0), _ptr(weight), _ptr(x), x.shape[0], x.shape[1],
+                                          float(eps), _is_bf16(y.dtype), _stream()), "norm_into_stream")
+
+
+def rms_norm_from_f32(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor) -> None:
+    """``out = weight * x / sqrt(mean(x^2) + eps)`` for a float32 ``x``, rounded once to ``out``'s type."""
+    _dense(x, "x", torch.float32, 2)
+    _dense(weight, "weight", torch.float32, 1)
+    _dense(out, "out", ndim=2)
+    _require(out.shape == x.shape and weight.shape[0] == x.shape[1], "out, x and weight disagree on the sizes")
+    _check(library().dli_rms_norm_from_f32(_ptr(x), _ptr(weight), _ptr(out), x.shape[0], x.shape[1], float(eps),
+                                           _is_bf16(out.dtype), _stream()), "rms_norm_from_f32")
+
+
+def softcap(y: torch.Tensor, cap: float) -> None:
+    """``y <- cap * tanh(y / cap)`` in place (float32)."""
+    _dense(y, "y", torch.float32)
+    _require(cap > 0, "the cap must be positive")
+    _check(library().dli_softcap(_ptr(y), y.numel(), float(cap), _stream()), "softcap")
+
+
+def token_shift(x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor,
+                positions: torch.Tensor, state_slots: torch.Tensor, out: torch.Tensor) -> None:
+    """``out[s, t] = x[t] + (x[t-1] - x[t]) * mu[s]`` for every mix ``s``; the row before an entry's
+    first row is the request's kept row, the first ``width`` floats of ``state[slot]`` (zeros at
+    position 0), which then receives the entry's last row. ``x`` float32 ``[n, width]``, ``mu`` float32
+    ``[mixes, width]``, ``state`` float32 ``[slots, >= width]``, ``out [mixes, n, width]``."""
+    _dense(x, "x", torch.float32, 2)
+    _dense(mu, "mu", torch.float32, 2)
+    _dense(out, "out", ndim=3)
+    n, width = x.shape
+    _require(mu.shape[1] == width and out.shape == (mu.shape[0], n, width), "x, mu and out disagree on the sizes")
+    _require(state.is_cuda and state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+             and state.shape[1] >= width, "state must be float32 [slots, >= width]")
+    for name, t in (("q_start", q_start), ("positions", positions), ("state_slots", state_slots)):
+        _dense(t, name, torch.int32, 1)
+    entries = state_slots.shape[0]
+    _require(q_start.shape[0] == entries + 1 and positions.shape[0] == n, "q_start/state_slots/positions disagree")
+    _check(library().dli_token_shift(_ptr(x), _ptr(mu), mu.shape[0], _ptr(state), state.stride(0), _ptr(q_start),
+                                     entries, _ptr(positions), _ptr(state_slots), _ptr(out), n, width,
+                                     _is_bf16(out.dtype), _stream()), "token_shift")
+
+
+def lowrank_out(t: torch.Tensor, w2: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                act: str = "tanh") -> None:
+    """``out = act(t) @ w2.T + bias`` in 32-bit: ``t`` float32 ``[n, rank]`` (rows contiguous, any row
+    stride), ``w2`` float32 ``[features, rank]``; ``act`` ``"tanh"`` or ``"none"``."""
+    _f32_rows(t, "t")
+    _dense(w2, "w2", torch.float32, 2)
+    _dense(out, "out", torch.float32, 2)
+    _require(act in ("tanh", "none"), "act must be 'tanh' or 'none'")
+    n, rank = t.shape
+    feats = w2.shape[0]
+    _require(w2.shape[1] == rank and out.shape == (n, feats), "t, w2 and out disagree on the sizes")
+    if bias is not None:
+        _dense(bias, "bias", torch.float32, 1)
+        _require(bias.shape[0] == feats, "bias length differs from rows of w2")
+    _check(library().dli_lowrank_out(_ptr(t), t.stride(0), _ptr(w2), _ptr(bias), _ptr(out), n, feats, rank,
+                                     1 if act == "tanh" else 0, _stream()), "lowrank_out")
+
+
+def qk_unit_cache(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, q_out: torch.Tensor,
+                  slots: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, q_heads: int, eps: float,
+                  mix: Optional[torch.Tensor] = None, v_first_in: Optional[torch.Tensor] = None,
+                  v_first_out: Optional[torch.Tensor] = None) -> None:
+    """From the float32 projections ``proj [n, >= ...]`` (q at ``q_off``, k at ``k_off``, v at
+    ``v_off``): q and k divided by their root mean square per head, ``q_out [n, q_heads*dim]``; with
+    ``mix`` (a float32 scalar on the device) ``v <- (1 - mix) v + mix v_first_in``; ``v_first_out``
+    receives this layer's v; k and v are written at each token's cache slot."""
+    _f32_rows(proj, "proj")
+    _dense(k_pages, "k_pages", ndim=4)
+    dtype = k_pages.dtype
+    pages, kv_heads, page_size, dim = k_pages.shape
+    _dense(v_pages, "v_pages", dtype, 4)
+    vdim = v_pages.shape[2]
+    _require(v_pages.shape == (pages, kv_heads, vdim, page_size), "v_pages must be [pages, kv_heads, vdim, page_size]")
+    n = proj.shape[0]
+    _dense(q_out, "q_out", dtype, 2)
+    _require(q_out.shape == (n, q_heads * dim), "q_out must be [n, q_heads*dim]")
+    _dense(slots, "slots", torch.int32, 1)
+    _require(slots.shape[0] == n, "slots differ from proj in rows")
+    for off, size in ((q_off, q_heads * dim), (k_off, kv_heads * dim), (v_off, kv_heads * vdim)):
+        _require(0 <= off and off + size <= proj.shape[1], "a projection lies outside proj's columns")
+    for t in (v_first_in, v_first_out):
+        if t is not None:
+            _dense(t, "v_first", torch.float32, 2)
+            _require(t.shape == (n, kv_heads * vdim), "v_first must be [n, kv_heads*vdim]")
+    if mix is not None:
+        _require(mix.is_cuda and mix.dtype == torch.float32 and mix.numel() == 1 and v_first_in is not None,
+                 "mix must be one float32 on the device, with v_first_in")
+    _check(library().dli_qk_unit_cache(
+        _ptr(proj), proj.stride(0), q_off, k_off, v_off, _ptr(q_out), _ptr(mix), _ptr(v_first_in), _ptr(v_first_out),
+        _ptr(slots), _ptr(k_pages), _ptr(v_pages), n, q_heads, kv_heads, dim, vdim, page_size, float(eps),
+        _is_bf16(dtype), _stream()), "qk_unit_cache")
+
+
+def attention_scored(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
+                     q_start: torch.Tensor, kv_len: torch.Tensor, block_tables: torch.Tensor,
+                     tile_entry: Optional[torch.Tensor], tile_q0: Optional[torch.Tensor], q_heads: int, scale: float,
+                     *, window: int = 0, chunk: int = 0, sink: bool = False, r1: Optional[torch.Tensor] = None,
+                     r2: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> None:
+    """Paged causal attention on the vector units (32-bit arithmetic) with changes to the scores
+    as parameters: ``window`` and ``chunk`` restrict the keys a query sees, ``r1, r2`` (float32
+    ``[q_heads]``) take ``r1 log(1 + r2 (p - j))`` off the scaled score, ``sink`` adds ``exp(0)`` to the
+    softmax's denominator, ``gate`` (float32 ``[tokens, q_heads*value_dim]``, rows contiguous)
+    multiplies the result by its sigmoid. Values may differ from keys in size (``v_pages``).
+    Without tile lists every entry is one row (a step of single tokens)."""
+    _dense(k_pages, "k_pages", ndim=4)
+    dtype = k_pages.dtype
+    _rows(q, "q", dtype)
+    _rows(out, "out", dtype)
+    pages, kv_heads, page_size, head_dim = k_pages.shape
+    _dense(v_pages, "v_pages", dtype, 4)
+    value_dim = v_pages.shape[2]
+    _require(v_pages.shape == (pages, kv_heads, value_dim, page_size),
+             "v_pages must be [pages, kv_heads, value_dim, page_size]")
+    _require(q.shape[1] == q_heads * head_dim and out.shape == (q.shape[0], q_heads * value_dim),
+             "q must be [tokens, q_heads*head_dim] and out [tokens, q_heads*value_dim]")
+    _require(q_heads % kv_heads == 0, "query heads are not a multiple of kv heads")
+    _require(max(head_dim, value_dim) <= 256, "heads of at most 256")
+    _dense(q_start, "q_start", torch.int32, 1)
+    _dense(kv_len, "kv_len", torch.int32, 1)
+    _dense(block_tables, "block_tables", torch.int32, 2)
+    entries = kv_len.shape[0]
+    _require(q_start.shape[0] == entries + 1 and block_tables.shape[0] >= entries,
+             "q_start/kv_len/block_tables disagree on the number of requests")
+    if tile_entry is None:
+        _require(tile_q0 is None and q.shape[0] == entries, "without tile lists every entry must be one row")
+        tiles = entries
+    else:
+        _dense(tile_entry, "tile_entry", torch.int32, 1)
+        _dense(tile_q0, "tile_q0", torch.int32, 1)
+        _require(tile_entry.shape == tile_q0.shape, "tile lists differ in length")
+        tiles = tile_entry.shape[0]
+    _require((r1 is None) == (r2 is None), "r1 and r2 come together")
+    for name, t in (("r1", r1), ("r2", r2)):
+        if t is not None:
+            _dense(t, name, torch.float32, 1)
+            _require(t.shape[0] == q_heads, f"{name} must hold one value per query head")
+    gate_stride = 0
+    if gate is not None:
+        _f32_rows(gate, "gate")
+        _require(gate.shape == out.shape, "gate differs from out in shape")
+        gate_stride = gate.stride(0)
+    _check(library().dli_attention_scored(
+        _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(q_start), _ptr(kv_len),
+        _ptr(block_tables), block_tables.stride(0), _ptr(tile_entry), _ptr(tile_q0), tiles, q_heads, kv_heads,
+        head_dim, value_dim, page_size, float(scale), int(window), int(chunk), int(bool(sink)), _ptr(r1), _ptr(r2),
+        _ptr(gate), gate_stride, _is_bf16(dtype), _stream()), "attention_scored")
+
+
+RULE_DELTA, RULE_BONUS = 0, 1
+
+
+def recurrent_scan_supports(dim: int) -> bool:
+    return bool(library().dli_recurrent_scan_supports(int(dim)))
+
+
+def recurrent_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, w_pre: torch.Tensor, g_pre: torch.Tensor,
+                   norm_w: torch.Tensor, eps: float, state: torch.Tensor, q_start: torch.Tensor,
+                   positions: torch.Tensor, state_slots: torch.Tensor, out: torch.Tensor, heads: int, dim: int,
+                   rule: int, a_pre: Optional[torch.Tensor] = None, a_bias: Optional[torch.Tensor] = None,
+                   bonus: Optional[torch.Tensor] = None) -> None:
+    """A matrix-state recurrence per request and head, with the per-head norm and the gate of its
+    output (``csrc/recurrent_scan.hip`` states both rules). ``r, k, v, w_pre, g_pre, a_pre`` are
+    float32 ``[n, heads*dim]`` with contiguous rows (any row stride); ``state`` is float32
+    ``[slots, >= heads*dim*dim]``, row ``state_slots[e]`` being entry ``e``'s; ``out [n, heads*dim]``
+    float32 or bfloat16."""
+    n, width = out.shape[0], heads * dim
+    for name, t in (("r", r), ("k", k), ("v", v), ("w_pre", w_pre), ("g_pre", g_pre), ("a_pre", a_pre)):
+        if t is not None:
+            _f32_rows(t, name)
+            _require(t.shape == (n, width), f"{name} must be [n, heads*dim]")
+    _rows(out, "out", out.dtype)
+    _require(out.shape[1] == width, "out must be [n, heads*dim]")
+    _require(recurrent_scan_supports(dim), f"the recurrence kernel takes heads of 16 to 128 in steps of 8 (16 above 64), not {dim}")
+    _dense(norm_w, "norm_w", torch.float32, 1)
+    _require(norm_w.shape[0] == width, "norm_w must hold heads*dim values")
+    _require(state.is_cuda and state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+             and state.shape[1] >= heads * dim * dim, "state must be float32 [slots, >= heads*dim*dim]")
+    for name, t in (("q_start", q_start), ("positions", positions), ("state_slots", state_slots)):
+        _dense(t, name, torch.int32, 1)
+    entries = state_slots.shape[0]
+    _require(q_start.shape[0] == entries + 1 and positions.shape[0] == n, "q_start/state_slots/positions disagree")
+    if rule == RULE_DELTA:
+        _require(a_pre is not None and a_bias is not None, "the delta rule needs a_pre and a_bias")
+        _dense(a_bias, "a_bias", torch.float32, 1)
+        _require(a_bias.shape[0] == width, "a_bias must hold heads*dim values")
+    else:
+        _require(rule == RULE_BONUS and bonus is not None, "the bonus rule needs bonus")
+        _dense(bonus, "bonus", torch.float32)
+        _require(bonus.numel() == width, "bonus must hold heads*dim values")
+    sa = a_pre.stride(0) if a_pre is not None else 0
+    _check(library().dli_recurrent_scan(
+        _ptr(r), r.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(w_pre), w_pre.stride(0), _ptr(a_pre), sa,
+        _ptr(a_bias), _ptr(g_pre), g_pre.stride(0), _ptr(bonus), _ptr(norm_w), float(eps), _ptr(state), state.stride(0),
+        _ptr(q_start), _ptr(positions), _ptr(state_slots), _ptr(out), out.stride(0), entries, heads, dim, int(rule),
+        _is_bf16(out.dtype), _stream()), "recurrent_scan")

@@ -13,4 +13,4 @@ __all__ = [
 ]
 
 # importing the modules registers the parts that ship with the engine
-from . import attention, block, embedding, feed_forward, head, norm, position  # noqa: E402,F401
+from . import attention, block, embedding, feed_forward, head, norm, position, recurrent, scored_attention  # noqa: E402,F401

@@ -161,6 +161,11 @@ class Embedding(Part):
     def forward(self, ids: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 
+    def forward_step(self, ctx: Any) -> torch.Tensor:
+        """The rows of a step: by default the rows of its token ids; an embedding that also
+        needs the positions (an absolute position encoding added to the rows) overrides this."""
+        return self.forward(ctx.token_ids)
+
     def table(self) -> torch.Tensor:
         """The ``[vocab, hidden]`` table, for a head that is tied to it."""
         raise NotImplementedError

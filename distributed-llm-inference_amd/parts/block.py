@@ -9,6 +9,7 @@ from typing import Any, Mapping, Optional
 import torch
 
 from .base import Block, DecodeStream, Part, Runtime
+from .linear import as_operand
 from .registry import register_part
 
 
@@ -64,3 +65,34 @@ class PreNormBlock(Block):
         kernel of the block may apply it while it writes the stream)."""
         parts["mixer"].forward_stream(stream, parts["mixer_norm"], ctx, cache, following=parts["feed_forward_norm"])
         parts["feed_forward"].forward_stream(stream, parts["feed_forward_norm"], ctx, following=following)
+
+
+@register_part("block", "output_norm")
+class OutputNormBlock(Block):
+    """Norms on the sublayers' outputs only, around a 32-bit residual stream:
+    ``x <- x + norm1(mixer(x))``, then ``x <- x + norm2(feed_forward(x))``; the sublayers read ``x``
+    itself. The feed-forward and its norm may be absent. ``x`` is float32 in both runtimes; each
+    norm is applied and added into the stream by one kernel (``Norm.add_normed``). The mixer gets
+    the stream as it is (what it feeds to its products it rounds itself); the feed-forward gets it
+    in the type that its products read."""
+
+    roles = ("mixer", "mixer_norm")
+
+    def __init__(self, runtime: Runtime) -> None:
+        super().__init__(runtime)
+
+    def graph_capturable(self, page_size: int) -> bool:
+        return True  # kernels on device arrays only
+
+    def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor], ctx: Any, cache: Any,
+                parts: Mapping[str, Part]) -> tuple[torch.Tensor, Optional[torch.Tensor]]:
+        if x.dtype != torch.float32:
+            raise RuntimeError("the output_norm block keeps a float32 residual stream")
+        if delta is not None:
+            from ..kernels import ops
+            ops.add(x, delta, x)
+        parts["mixer_norm"].add_normed(x, parts["mixer"].forward(x, ctx, cache))
+        if "feed_forward" in parts:
+            y = parts["feed_forward"].forward(as_operand(self.rt, x), ctx)
+            parts["feed_forward_norm"].add_normed(x, y)
+        return x, None

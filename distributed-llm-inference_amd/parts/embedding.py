@@ -2,8 +2,9 @@
 
 from __future__ import annotations
 
-from typing import Mapping
+from typing import Any, Mapping, Optional
 
+import numpy as np
 import torch
 
 from ..kernels import ops
@@ -46,3 +47,42 @@ class TokenEmbedding(Embedding):
         ssq = torch.empty(1, n, device=self.rt.device, dtype=torch.float32)
         ops.embedding_ssq(self.table(), ids, out, ssq)
         return DecodeStream(out, ssq)
+
+
+@register_part("embedding", "sinusoidal_token_embedding")
+class SinusoidalTokenEmbedding(TokenEmbedding):
+    """Token rows plus an absolute sinusoidal position vector, into a 32-bit residual stream:
+    ``x[t] = table[id] + pe(p)`` with ``pe[2i] = sin(p base^(-2i/width))`` and ``pe[2i+1]`` the cosine of
+    the same angle. The frequencies are made once on the host in double precision and rounded to
+    float32; angles and sums are 32-bit on the device. The rows are float32 whatever the runtime's
+    type (the table itself has the runtime's type, so a tied head can read it)."""
+
+    def __init__(self, runtime: Runtime, *, vocab_size: int, hidden_size: int, base: float = 10000.0,
+                 weight_name: str = "weight") -> None:
+        super().__init__(runtime, vocab_size=vocab_size, hidden_size=hidden_size)
+        self.base, self.weight_name = float(base), weight_name
+        self._inv_freq: Optional[torch.Tensor] = None
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        return {self.weight_name: WeightSpec((self.vocab_size, self.hidden_size))}
+
+    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        self.weight = tensors[self.weight_name]
+
+    def finalize(self) -> None:
+        pairs = (self.hidden_size + 1) // 2
+        inv = np.power(self.base, -2.0 * np.arange(pairs, dtype=np.float64) / self.hidden_size).astype(np.float32)
+        self._inv_freq = torch.from_numpy(inv).to(self.rt.device)
+
+    def streams(self, ctx) -> bool:
+        return False  # the fused decode kernels keep a stream of the runtime's type
+
+    def forward(self, ids: torch.Tensor) -> torch.Tensor:
+        raise RuntimeError("this embedding needs the positions of the step: call forward_step(ctx)")
+
+    def forward_step(self, ctx: Any) -> torch.Tensor:
+        if self._inv_freq is None:
+            self.finalize()
+        out = torch.empty(ctx.token_ids.shape[0], self.hidden_size, device=self.rt.device, dtype=torch.float32)
+        ops.embed_sinusoid(self.table(), ctx.token_ids, ctx.positions, self._inv_freq, out)
+        return out

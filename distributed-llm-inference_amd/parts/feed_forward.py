@@ -17,9 +17,15 @@ from .spec import WeightSpec
 
 @register_part("feed_forward", "gated_mlp")
 class GatedMLP(FeedForward):
+    NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
+
     def __init__(self, runtime: Runtime, *, hidden_size: int, intermediate_size: int,
-                 activation: str = "silu", bias: bool = False) -> None:
+                 activation: str = "silu", bias: bool = False, names: Optional[Mapping[str, str]] = None) -> None:
         super().__init__(runtime)
+        # checkpoint names of the three matrices below the part's prefix, where they are not the usual ones
+        self.names = {**self.NAMES, **dict(names or {})}
+        if bias and names:
+            raise ValueError("gated_mlp: other tensor names are taken for the matrices only")
         if activation != "silu":
             raise ValueError(f"gated_mlp has no kernel for activation {activation!r} (only 'silu')")
         self.hidden_size, self.intermediate_size, self.bias = hidden_size, intermediate_size, bias
@@ -31,16 +37,16 @@ class GatedMLP(FeedForward):
 
     def weight_specs(self) -> dict[str, WeightSpec]:
         h, i = self.hidden_size, self.intermediate_size
-        specs = {"gate_proj.weight": WeightSpec((i, h)), "up_proj.weight": WeightSpec((i, h)),
-                 "down_proj.weight": WeightSpec((h, i))}
+        specs = {self.names["gate"]: WeightSpec((i, h)), self.names["up"]: WeightSpec((i, h)),
+                 self.names["down"]: WeightSpec((h, i))}
         if self.bias:
             specs.update({"gate_proj.bias": WeightSpec((i,)), "up_proj.bias": WeightSpec((i,)),
                           "down_proj.bias": WeightSpec((h,))})
         return specs
 
     def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
-        self.w_gate_up = torch.cat([tensors["gate_proj.weight"], tensors["up_proj.weight"]], 0).contiguous()
-        self.w_down = tensors["down_proj.weight"]
+        self.w_gate_up = torch.cat([tensors[self.names["gate"]], tensors[self.names["up"]]], 0).contiguous()
+        self.w_down = tensors[self.names["down"]]
         if self.bias:
             self.b_gate_up = torch.cat([tensors["gate_proj.bias"], tensors["up_proj.bias"]], 0).contiguous()
             self.b_down = tensors["down_proj.bias"]

@@ -16,9 +16,11 @@ from .spec import WeightSpec
 
 @register_part("head", "linear_head")
 class LinearHead(Head):
-    def __init__(self, runtime: Runtime, *, vocab_size: int, hidden_size: int, tied: bool) -> None:
+    def __init__(self, runtime: Runtime, *, vocab_size: int, hidden_size: int, tied: bool,
+                 softcap: float = 0.0) -> None:
         super().__init__(runtime)
         self.vocab_size, self.hidden_size, self.tied = vocab_size, hidden_size, tied
+        self.softcap = float(softcap)  # > 0: logits <- softcap * tanh(logits / softcap)
         self.weight: Optional[torch.Tensor] = None
         self.weight_tiled: Optional[torch.Tensor] = None
 
@@ -42,6 +44,12 @@ class LinearHead(Head):
     FEW_ROWS = 16  # up to here the decode product streams the table faster than the library does
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        logits = self._logits(x)
+        if self.softcap > 0:
+            ops.softcap(logits, self.softcap)
+        return logits
+
+    def _logits(self, x: torch.Tensor) -> torch.Tensor:
         rows = x.shape[0]
         if (self.rt.is_bf16 and 0 < rows <= self.FEW_ROWS and x.dtype == torch.bfloat16
                 and ops.skinny_gemm_supports(rows, self.hidden_size, self.rt.dtype)):
@@ -62,7 +70,7 @@ class LinearHead(Head):
         return out
 
     def streams(self, ctx) -> bool:
-        return self.rt.is_bf16 and (ctx.num_tokens > self.FEW_ROWS
+        return self.softcap == 0 and self.rt.is_bf16 and (ctx.num_tokens > self.FEW_ROWS
                                     or ops.skinny_gemm_supports(ctx.num_tokens, self.hidden_size, self.rt.dtype))
 
     def forward_stream(self, stream: DecodeStream, norm: Norm, argmax: Optional[ArgmaxStage] = None) -> torch.Tensor:

@@ -76,3 +76,45 @@ def finish_residual(rt: Runtime, stream: DecodeStream, partial: torch.Tensor, bi
         stream.wrote(ssq, normed, following)
     else:
         stream.wrote(ops.mid_finish_residual(partial, stream.x, bias))
+
+
+def as_operand(rt: Runtime, x: torch.Tensor) -> torch.Tensor:
+    """``x`` in the type that the runtime's products read: a 32-bit residual stream is rounded to
+    bfloat16 when serving and used as it is on the 32-bit path."""
+    if x.dtype == rt.dtype:
+        return x
+    if x.dtype != torch.float32:
+        raise ops.KernelArgumentError(f"an operand of type {x.dtype} in a runtime of {rt.dtype}")
+    out = rt.empty(*x.shape)
+    ops.cast_from_f32(x, out)
+    return out
+
+
+F32_FEW_ROWS = 16  # up to here the few-row product streams the weights faster than the library does
+
+
+def linear_f32(rt: Runtime, x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``x [n, k] @ weight[m, k].T -> float32 [n, m]``: the 32-bit sums of the product as they are,
+    for what is computed in 32-bit after a projection (recurrences, norms, gates). ``out`` may be a
+    view of some columns of a wider float32 matrix."""
+    n, m = x.shape[0], weight.shape[0]
+    if out is None:
+        out = torch.empty(n, m, device=rt.device, dtype=torch.float32)
+    if n == 0:
+        return out
+    if rt.dtype == torch.float32:
+        ops.gemm_f32(x, weight, out)
+        return out
+    k = x.shape[1]
+    if (n <= F32_FEW_ROWS and ops.skinny_gemm_supports(n, k, x.dtype) and x.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0 and out.data_ptr() % 16 == 0 and weight.is_contiguous()):
+        ops.skinny_gemm(x, weight, epilogue=ops.SKINNY_F32, out=out)
+        return out
+    if not ops.gemm_bf16(x, weight, out):
+        # a shape for which the direct call finds no kernel: the same library through torch
+        # (bfloat16 result, widened)
+        tmp = torch.mm(x, weight.t())
+        wide = torch.empty(n, m, device=rt.device, dtype=torch.float32)
+        ops.to_float(tmp, wide)
+        out.copy_(wide)
+    return out

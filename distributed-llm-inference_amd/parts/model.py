@@ -20,7 +20,7 @@ from .registry import build_part
 from .spec import ModelSpec, WeightSpec
 
 # importing the modules registers the built-in parts
-from . import attention, block, embedding, feed_forward, head, norm, position  # noqa: F401,E402
+from . import attention, block, embedding, feed_forward, head, norm, position, recurrent, scored_attention  # noqa: F401,E402
 
 
 @dataclass
@@ -193,7 +193,7 @@ class Model:
         ctx.begin_forward()
         if self._streams(ctx):
             return self._forward_stream(ctx, caches)
-        x = self.embedding.forward(ctx.token_ids)
+        x = self.embedding.forward_step(ctx)
         delta: Optional[torch.Tensor] = None
         native = self._native_blocks(caches) if self.rt.is_bf16 and self.native_steps and ctx.num_tokens > 0 else None
         if native is not None:

@@ -15,19 +15,19 @@ from .spec import WeightSpec
 
 @register_part("norm", "rms_norm")
 class RMSNorm(Norm):
-    def __init__(self, runtime: Runtime, *, width: int, eps: float) -> None:
+    def __init__(self, runtime: Runtime, *, width: int, eps: float, weight_name: str = "weight") -> None:
         super().__init__(runtime)
-        self.width, self.eps = width, float(eps)
+        self.width, self.eps, self.weight_name = width, float(eps), weight_name
         self.weight: torch.Tensor | None = None
 
     def graph_capturable(self, page_size: int) -> bool:
         return True  # kernels on device arrays only
 
     def weight_specs(self) -> dict[str, WeightSpec]:
-        return {"weight": WeightSpec((self.width,), role="float32", init="norm")}
+        return {self.weight_name: WeightSpec((self.width,), role="float32", init="norm")}
 
     def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
-        self.weight = tensors["weight"]
+        self.weight = tensors[self.weight_name]
 
     def fused_params(self) -> tuple[torch.Tensor, float]:
         """Weight and eps, for a consumer that computes this norm inside its own kernel."""
@@ -41,7 +41,20 @@ class RMSNorm(Norm):
             return None
         return {"kind": "rms_norm", "w": w, "eps": self.eps, "width": self.width}
 
+    def add_normed(self, x: torch.Tensor, y: torch.Tensor) -> None:
+        """``x += norm(y)``: the norm on a sublayer's output, added into a 32-bit residual stream
+        ``x`` in one kernel (statistics, product and sum in 32-bit; ``y`` float32 or bfloat16)."""
+        ops.norm_into_stream(y, self.weight, self.eps, x)
+
     def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if x.dtype == torch.float32 and self.rt.is_bf16:
+            # a 32-bit residual stream in a bfloat16 runtime: normalised in 32-bit and rounded once,
+            # to the type that the product after the norm reads
+            if delta is not None:
+                ops.add(x, delta, x)
+            out = self.rt.empty(*x.shape)
+            ops.rms_norm_from_f32(x, self.weight, self.eps, out)
+            return out
         out = torch.empty_like(x)
         if delta is None:
             ops.rms_norm(x, self.weight, self.eps, out)

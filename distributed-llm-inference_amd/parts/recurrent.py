@@ -1,0 +1,157 @@
+"""Mixers that carry a matrix state per head from token to token instead of a cache of keys:
+``general_delta`` (a generalized delta rule) and ``wkv`` (decayed sums with a bonus for the current
+token and token shift). The state lives in 32-bit in the request's state slot
+(:class:`StateSpec`), starts at zero at position 0, and is all that a step leaves for the next.
+
+Both run their projections as products of the runtime's type with 32-bit sums, and everything
+after them in 32-bit: decays, rates, unit keys, the recurrence, the per-head norm of its output
+and the gate (``csrc/recurrent_scan.hip``). The decay's pre-activation is a low-rank projection,
+``W2 tanh(W1 h) + w0``, whose second half is 32-bit; its rank is read off the checkpoint's tensor.
+"""
+
+from __future__ import annotations
+
+from typing import Any, Mapping, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import Mixer, Runtime, StateSpec
+from .linear import as_operand, linear_f32
+from .registry import register_part
+from .spec import WeightSpec
+
+
+def default_rank(hidden_size: int) -> int:
+    """The rank that random-weights mode gives a low-rank projection when nothing names one."""
+    return max(8, min(64, hidden_size // 16 // 8 * 8))
+
+
+class _MatrixStateMixer(Mixer):
+    """What the two rules share: sizes, the state, the decay's low-rank projection and the output."""
+
+    rule = -1
+
+    def __init__(self, runtime: Runtime, *, hidden_size: int, num_heads: int, head_dim: int, norm_eps: float = 1e-6,
+                 decay_rank: Optional[int] = None) -> None:
+        super().__init__(runtime)
+        if num_heads < 1 or head_dim < 1:
+            raise ValueError("heads and their size must be positive")
+        self.hidden_size, self.num_heads, self.head_dim = hidden_size, num_heads, head_dim
+        self.norm_eps, self.decay_rank = float(norm_eps), decay_rank
+        self.width = num_heads * head_dim
+        self.w2 = self.w0 = self.norm_w = self.w_o = None
+
+    def _shared_specs(self) -> dict[str, WeightSpec]:
+        h, c = self.hidden_size, self.width
+        rank = self.decay_rank if self.decay_rank else -1
+        drawn = self.decay_rank or default_rank(h)
+        return {"w1": WeightSpec((rank, h), drawn_shape=(drawn, h)),
+                "w2": WeightSpec((c, rank), role="float32", drawn_shape=(c, drawn)),
+                "w0": WeightSpec((c,), role="float32"), "norm": WeightSpec((c,), role="float32", init="norm"),
+                "o": WeightSpec((h, c))}
+
+    def _load_shared(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        if tensors["w1"].shape[0] != tensors["w2"].shape[1]:
+            raise ValueError(f"{self.prefix}w1 and {self.prefix}w2 disagree on the rank of the decay's projection")
+        self.w2, self.w0 = tensors["w2"].contiguous(), tensors["w0"]
+        self.norm_w, self.w_o = tensors["norm"], tensors["o"]
+
+    def graph_capturable(self, page_size: int) -> bool:
+        return True  # kernels on the context's device arrays only; padding rows write the spare slot
+
+    def _check(self, cache: Any) -> torch.Tensor:
+        if cache is None or cache.kind != "state" or not cache.writable:
+            raise RuntimeError(f"{self.kind} needs a state of its own")
+        if not ops.recurrent_scan_supports(self.head_dim):
+            raise ops.KernelArgumentError(f"the recurrence kernel does not take heads of {self.head_dim}")
+        return cache.state.view(cache.state.shape[0], -1)
+
+
+@register_part("mixer", "general_delta")
+class GeneralDelta(_MatrixStateMixer):
+    """Per head, with ``u = k / sqrt(sum k^2 + 1e-6)``, ``w = exp(-exp(-1/2) sigmoid(W2 tanh(W1 h) + w0))`` and
+    ``a = sigmoid(W_a h + b_a)`` per key channel: ``S <- diag(w) S - (a * u)(u^T S) + k v^T`` (both terms read
+    the old state), ``o = S^T r``; then ``o / rms(o) * norm * sigmoid(W_g h)`` and the output product."""
+
+    rule = ops.RULE_DELTA
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        h, c = self.hidden_size, self.width
+        specs = {n: WeightSpec((c, h)) for n in ("r", "k", "v", "g", "a")}
+        specs["a.b"] = WeightSpec((c,), role="float32")
+        specs.update(self._shared_specs())
+        return specs
+
+    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        # one product for everything that reads h: r, k, v, g, a, and the first half of the decay's
+        self.w_in = torch.cat([tensors[n] for n in ("r", "k", "v", "g", "a", "w1")], dim=0).contiguous()
+        self.rank = tensors["w1"].shape[0]
+        self.a_bias = tensors["a.b"]
+        self._load_shared(tensors)
+
+    def cache_spec(self) -> StateSpec:
+        return StateSpec((self.num_heads * self.head_dim * self.head_dim,), torch.float32)
+
+    def forward(self, x: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:
+        state = self._check(cache)
+        n, c = x.shape[0], self.width
+        proj = linear_f32(self.rt, as_operand(self.rt, x), self.w_in)
+        r, k, v, g, a = (proj[:, i * c:(i + 1) * c] for i in range(5))
+        w_pre = torch.empty(n, c, device=self.rt.device, dtype=torch.float32)
+        ops.lowrank_out(proj[:, 5 * c:5 * c + self.rank], self.w2, self.w0, w_pre, act="tanh")
+        out = self.rt.empty(n, c)
+        ops.recurrent_scan(r, k, v, w_pre, g, self.norm_w, self.norm_eps, state, ctx.q_start, ctx.positions,
+                           ctx.state_slots, out, self.num_heads, self.head_dim, self.rule, a_pre=a, a_bias=self.a_bias)
+        return linear_f32(self.rt, out, self.w_o)
+
+
+@register_part("mixer", "wkv")
+class WKV(_MatrixStateMixer):
+    """Token shift, then per head ``o = (S + diag(u) k v^T)^T r`` and ``S <- diag(w) S + k v^T`` with
+    ``w = exp(-exp(W2 tanh(W1 m_w) + w0))``; r, k, v, the gate and the decay each read a mix of their
+    own, ``m_s = h + (h_prev - h) * mu_s``, of the row with the row before it (zeros before position
+    0; the last row of a step is kept in the state beside S). Then ``o / rms(o) * norm * silu(W_g m_g)``
+    and the output product."""
+
+    rule = ops.RULE_BONUS
+    MIXES = ("r", "k", "v", "g", "w")
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        h, c = self.hidden_size, self.width
+        specs = {n: WeightSpec((c, h)) for n in ("r", "k", "v", "g")}
+        specs.update({f"mu.{s}": WeightSpec((h,), role="float32") for s in self.MIXES})
+        specs["u"] = WeightSpec((self.num_heads, self.head_dim), role="float32")
+        specs.update(self._shared_specs())
+        return specs
+
+    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        self.w = {n: tensors[n] for n in ("r", "k", "v", "g")}
+        self.w1 = tensors["w1"]
+        self.rank = self.w1.shape[0]
+        self.mu = torch.stack([tensors[f"mu.{s}"] for s in self.MIXES], dim=0).contiguous()
+        self.bonus = tensors["u"].contiguous()
+        self._load_shared(tensors)
+
+    def cache_spec(self) -> StateSpec:
+        # the row before the next step's first row, then S
+        return StateSpec((self.hidden_size + self.num_heads * self.head_dim * self.head_dim,), torch.float32)
+
+    def forward(self, x: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:
+        state = self._check(cache)
+        if x.dtype != torch.float32:
+            raise RuntimeError("wkv shifts the rows of a float32 residual stream")
+        n, c, h = x.shape[0], self.width, self.hidden_size
+        mixes = self.rt.empty(len(self.MIXES), n, h)
+        ops.token_shift(x, self.mu, state, ctx.q_start, ctx.positions, ctx.state_slots, mixes)
+        proj = torch.empty(n, 4 * c + self.rank, device=self.rt.device, dtype=torch.float32)
+        for i, name in enumerate(("r", "k", "v", "g")):
+            linear_f32(self.rt, mixes[i], self.w[name], out=proj[:, i * c:(i + 1) * c])
+        linear_f32(self.rt, mixes[4], self.w1, out=proj[:, 4 * c:])
+        r, k, v, g = (proj[:, i * c:(i + 1) * c] for i in range(4))
+        w_pre = torch.empty(n, c, device=self.rt.device, dtype=torch.float32)
+        ops.lowrank_out(proj[:, 4 * c:], self.w2, self.w0, w_pre, act="tanh")
+        out = self.rt.empty(n, c)
+        ops.recurrent_scan(r, k, v, w_pre, g, self.norm_w, self.norm_eps, state[:, h:], ctx.q_start, ctx.positions,
+                           ctx.state_slots, out, self.num_heads, self.head_dim, self.rule, bonus=self.bonus)
+        return linear_f32(self.rt, out, self.w_o)

@@ -1,0 +1,144 @@
+"""Grouped-query attention over the paged cache whose scores are changed by parameters: unit-RMS
+queries and keys, a per-head logarithmic distance penalty, a chunked mask, a softmax with a sink,
+value mixing across layers, and a sigmoid output gate. Each is a parameter that is off by default,
+so another design may take any subset.
+
+Order of work for the rows ``h`` of a step (``x`` may be a 32-bit residual stream; the products read
+it in the runtime's type):
+
+1. one product gives q, k, v and the gate's pre-activation (the checkpoint's matrices stacked at
+   load), as 32-bit sums;
+2. one kernel divides every head's q and k by its root mean square over ``dim`` (``qk_unit``), mixes
+   v with the values that the first such layer of the step computed for the same token
+   (``value_mix``: ``v <- (1 - m) v + m v_first``), and writes k and the mixed v into the cache pages;
+3. the attention kernel: ``s_ij = scale (q_i . k_j) - r1_h log(1 + r2_h (i - j))`` for ``j <= i`` in
+   the same chunk of ``chunk`` positions (counted from the request's position 0), weights
+   ``exp(s_ij) / (sink + sum_j exp(s_ij))`` with ``sink = 1`` (a key of score 0 that has no value),
+   the result multiplied by ``sigmoid(gate)``;
+4. the output product, 32-bit sums.
+
+Scores, weights, norms and the mixing are 32-bit; keys and values are cached in the runtime's type.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Any, Mapping, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import Mixer, PagedKVSpec, Runtime
+from .linear import as_operand, linear_f32
+from .registry import register_part
+from .spec import WeightSpec
+
+
+@register_part("mixer", "scored_attention")
+class ScoredAttention(Mixer):
+    VALUE_MIX = ("none", "source", "mix")
+
+    def __init__(self, runtime: Runtime, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 value_dim: Optional[int] = None, scale: Optional[float] = None, qk_unit: bool = True,
+                 norm_eps: float = 1e-6, distance_penalty: bool = False, chunk: int = 0, window: int = 0,
+                 sink: bool = False, output_gate: bool = False, value_mix: str = "none",
+                 value_mix_key: str = "first_values", names: Optional[Mapping[str, str]] = None) -> None:
+        super().__init__(runtime)
+        if num_heads < 1 or num_kv_heads < 1 or num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} query heads do not group onto {num_kv_heads} kv heads")
+        value_dim = head_dim if value_dim is None else value_dim
+        if not 0 < head_dim <= 256 or not 0 < value_dim <= 256:
+            raise ops.KernelArgumentError(f"attention takes heads of 1 to 256, not {head_dim} / {value_dim}")
+        if value_mix not in self.VALUE_MIX:
+            raise ValueError(f"value_mix must be one of {self.VALUE_MIX}")
+        if chunk < 0 or window < 0:
+            raise ValueError("chunk and window must not be negative")
+        self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
+        self.head_dim, self.value_dim = head_dim, value_dim
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
+        self.qk_unit, self.norm_eps = bool(qk_unit), float(norm_eps)
+        self.distance_penalty, self.chunk, self.window = bool(distance_penalty), int(chunk), int(window)
+        self.sink, self.output_gate = bool(sink), bool(output_gate)
+        self.value_mix, self.value_mix_key = value_mix, value_mix_key
+        if not self.qk_unit:
+            raise ValueError("scored_attention caches unit keys: qk_unit=False has no kernel")
+        self.names = {"q": "q", "k": "k", "v": "v", "g": "g", "o": "o", "mix": "vmix", "r1": "r1", "r2": "r2",
+                      **dict(names or {})}
+        self.w_in = self.w_o = self.mix = self.r1 = self.r2 = None
+
+    # -- sizes of the stacked projection's parts
+    @property
+    def _q(self) -> int:
+        return self.num_heads * self.head_dim
+
+    @property
+    def _k(self) -> int:
+        return self.num_kv_heads * self.head_dim
+
+    @property
+    def _v(self) -> int:
+        return self.num_kv_heads * self.value_dim
+
+    @property
+    def _o(self) -> int:
+        return self.num_heads * self.value_dim
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        n, h = self.names, self.hidden_size
+        specs = {n["q"]: WeightSpec((self._q, h)), n["k"]: WeightSpec((self._k, h)), n["v"]: WeightSpec((self._v, h)),
+                 n["o"]: WeightSpec((h, self._o))}
+        if self.output_gate:
+            specs[n["g"]] = WeightSpec((self._o, h))
+        if self.distance_penalty:
+            specs[n["r1"]] = WeightSpec((self.num_heads,), role="float32", init="norm")
+            specs[n["r2"]] = WeightSpec((self.num_heads,), role="float32", init="norm")
+        if self.value_mix != "none":
+            # the source layer's file carries the scalar too, unused
+            specs[n["mix"]] = WeightSpec((), role="float32")
+        return specs
+
+    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        n = self.names
+        stacked = [tensors[n["q"]], tensors[n["k"]], tensors[n["v"]]] + ([tensors[n["g"]]] if self.output_gate else [])
+        self.w_in = torch.cat(stacked, dim=0).contiguous()
+        self.w_o = tensors[n["o"]]
+        if self.distance_penalty:
+            self.r1, self.r2 = tensors[n["r1"]].contiguous(), tensors[n["r2"]].contiguous()
+        if self.value_mix == "mix":
+            self.mix = tensors[n["mix"]].reshape(1).contiguous()
+
+    def cache_spec(self) -> PagedKVSpec:
+        return PagedKVSpec(self.num_kv_heads, self.head_dim, self.window,
+                           None if self.value_dim == self.head_dim else self.value_dim)
+
+    def graph_capturable(self, page_size: int) -> bool:
+        return True  # a step of single tokens is read through the context's device arrays alone
+
+    def forward(self, x: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:
+        if cache is None or cache.kind != "paged" or not cache.writable:
+            raise RuntimeError("scored_attention needs a paged cache of its own")
+        grp = ctx.groups[cache.group]
+        n = x.shape[0]
+        proj = linear_f32(self.rt, as_operand(self.rt, x), self.w_in)
+        q = self.rt.empty(n, self._q)
+        first_in = first_out = None
+        if self.value_mix == "source":
+            first_out = ctx.memo(("value mix", self.value_mix_key),
+                                 lambda: torch.empty(n, self._v, device=self.rt.device, dtype=torch.float32))
+        elif self.value_mix == "mix":
+            first_in = ctx._memo.get(("value mix", self.value_mix_key))
+            if first_in is None or first_in.shape != (n, self._v):
+                raise RuntimeError("value mixing needs an earlier layer of the step that keeps its values, of the same size")
+        ops.qk_unit_cache(proj, 0, self._q, self._q + self._k, q, grp.slots, cache.k_pages, cache.v_pages,
+                          self.num_heads, self.norm_eps, mix=self.mix if self.value_mix == "mix" else None,
+                          v_first_in=first_in, v_first_out=first_out)
+        out = self.rt.empty(n, self._o)
+        gate = proj[:, self._q + self._k + self._v:] if self.output_gate else None
+        if ctx.num_decode == ctx.num_entries:
+            tiles = (None, None)  # every entry is one row: nothing is derived from the step's lengths on the host
+        else:
+            tiles = ctx.q_tiles(ops.attention_generic_tile_rows(max(self.head_dim, self.value_dim)))
+        ops.attention_scored(q, cache.k_pages, cache.v_pages, out, ctx.q_start, ctx.kv_len, grp.block_tables,
+                             tiles[0], tiles[1], self.num_heads, self.scale, window=self.window, chunk=self.chunk,
+                             sink=self.sink, r1=self.r1, r2=self.r2, gate=gate)
+        return linear_f32(self.rt, out, self.w_o)

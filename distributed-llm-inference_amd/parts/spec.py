@@ -28,10 +28,23 @@ class WeightSpec:
     role: str = "matrix"
     optional: bool = False
     init: str = "normal"  # random-weights mode: "normal" (std 0.02), "ones", "zeros", "norm"
+    # A size that only the checkpoint gives is -1 in ``shape`` (any size fits; the part reads it off
+    # the tensor it receives); ``drawn_shape`` is then the shape that random-weights mode draws.
+    drawn_shape: Optional[tuple[int, ...]] = None
 
     def __post_init__(self) -> None:
         if self.role not in ("matrix", "float32", "int32"):
             raise ValueError(f"unknown weight role {self.role!r}")
+        if any(n == -1 for n in self.shape) and (self.drawn_shape is None or not self.fits(self.drawn_shape)):
+            raise ValueError("a shape with a free size needs a drawn_shape that fits it")
+
+    def fits(self, shape: tuple[int, ...]) -> bool:
+        """Whether a tensor of ``shape`` is what this spec asks for."""
+        return len(shape) == len(self.shape) and all(want in (-1, got) for want, got in zip(self.shape, shape))
+
+    @property
+    def shape_to_draw(self) -> tuple[int, ...]:
+        return tuple(self.drawn_shape) if self.drawn_shape is not None else tuple(self.shape)
 
 
 @dataclass(frozen=True)

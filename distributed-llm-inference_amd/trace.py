@@ -28,6 +28,7 @@ from typing import Any, Optional, Sequence, TextIO
 import numpy as np
 
 PAGE_SIZE = 16  # divides the 64 tokens that each request's count is rounded up to
+MAX_LIVE = 4    # requests that are live at a time: that many state slots, which are used again
 
 
 class TraceError(ValueError):
@@ -144,11 +145,16 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
                    help="most tokens that live requests hold at any time (each rounded up to 64)")
     p.add_argument("--page-size", type=int, default=PAGE_SIZE,
                    help=f"token slots of a cache page (default {PAGE_SIZE}; the pool is --max-tokens / this)")
+    p.add_argument("--max-live", type=int, default=MAX_LIVE,
+                   help=f"most requests that are live at a time (default {MAX_LIVE}): the number of state slots")
     args = p.parse_args(argv)
     try:
         if args.page_size < 1 or 64 % args.page_size:
             raise TraceError("--page-size must divide the 64 tokens that a request's count is rounded up to")
-        runner = TraceRunner(args.model, args.dtype, args.out, args.max_tokens, page_size=args.page_size)
+        if args.max_live < 1:
+            raise TraceError("--max-live must be positive")
+        runner = TraceRunner(args.model, args.dtype, args.out, args.max_tokens, page_size=args.page_size,
+                             max_live=args.max_live)
         runner.replay(sys.stdin, sys.stdout)
     except Exception as exc:  # one clear line, non-zero exit
         print(f"trace_run: {type(exc).__name__}: {exc}", file=sys.stderr, flush=True)

@@ -136,7 +136,7 @@ def load_model(model_dir: str | Path, *, dtype: str | torch.dtype = "bfloat16",
         unexpected = sorted(n for n in where if n not in expected)
         bad_shape = sorted(
             f"{n}: file {list(where[n].shape_of(n))}, model {list(s.shape)}"
-            for n, s in expected.items() if n in where and where[n].shape_of(n) != tuple(s.shape))
+            for n, s in expected.items() if n in where and not s.fits(tuple(where[n].shape_of(n))))
         if missing:
             problems.append(f"missing tensors: {_short(missing)}")
         if unexpected:

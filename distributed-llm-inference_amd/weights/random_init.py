@@ -82,18 +82,18 @@ def write_random_model(out_dir: str | Path, config: Mapping[str, Any] | Any, *, 
     tensors: dict[str, tuple[str, np.ndarray]] = {}
     for name, spec in model.weight_specs().items():
         if spec.role == "int32":
-            tensors[name] = ("I32", np.zeros(spec.shape, np.int32))
+            tensors[name] = ("I32", np.zeros(spec.shape_to_draw, np.int32))
             continue
         if torch.device(device).type != "cpu":
-            t = _drawn_on_device(name, tuple(spec.shape), spec.init, seed, std, norm_jitter, torch.device(device))
+            t = _drawn_on_device(name, spec.shape_to_draw, spec.init, seed, std, norm_jitter, torch.device(device))
             if storage == "bfloat16":
                 tensors[name] = ("BF16", t.to(torch.bfloat16).view(torch.int16).cpu().numpy().view(np.uint16))
             else:
                 tensors[name] = ("F32", t.cpu().numpy())
             continue
-        values = random_tensor(name, tuple(spec.shape), spec.init, seed, std, norm_jitter)
+        values = random_tensor(name, spec.shape_to_draw, spec.init, seed, std, norm_jitter)
         if storage == "bfloat16":
-            tensors[name] = ("BF16", float32_to_bfloat16_bits(values).reshape(spec.shape))
+            tensors[name] = ("BF16", float32_to_bfloat16_bits(values).reshape(spec.shape_to_draw))
         else:
             tensors[name] = ("F32", values)
     out = Path(out_dir)
