@@ -241,6 +241,63 @@ def serving_run(raw, dtype, workload, budget, decode_steps, rounds=2, model=None
     return result, cfg
 
 
+def makodra_shape(width, heads, kv_heads, ff, layers, vocab, chunk):
+    """A Makodra of sizes that resemble a real model's layers: heads of 64, every fourth layer an
+    attention layer (the first and every later one mixing values), two delta-rule layers and one
+    wkv layer between, a gated feed-forward in every layer."""
+    def layer(kind):
+        if kind == "attention":
+            mixer = {"heads": heads, "kv_heads": kv_heads, "dim": 64, "vdim": 64, "scale": 0.125, "v_mix": True,
+                     "mask": {"size": chunk}}
+        else:
+            mixer = {"heads": heads, "dim": 64, "rank": 64}
+        return {"type": kind, "mixer": mixer, "mlp": {"kind": "dense", "ff": ff}}
+    order = ["attention", "general_delta", "general_delta", "wkv"]
+    return {"architecture": "Makodra", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+            "layers": [layer(order[i % 4]) for i in range(layers)]}
+
+
+DESIGN_SIZES = {  # width, heads (of 64), kv heads, feed-forward, layers, vocabulary, attention chunk
+    "1024": (1024, 16, 4, 4096, 8, 32000, 1024),
+    "2048": (2048, 32, 8, 8192, 8, 32000, 2048),
+}
+
+
+def design_compare(args):
+    """Prefill and decode throughput of Makodra beside the Llama decoder at equal width, heads,
+    feed-forward, layers and vocabulary (random weights), each through the engine's own step loop."""
+    import gc
+
+    import torch
+
+    out = {}
+    for name in args.design_sizes.split(","):
+        width, heads, kv_heads, ff, layers, vocab, chunk = DESIGN_SIZES[name]
+        shapes = {
+            "makodra": makodra_shape(width, heads, kv_heads, ff, layers, vocab, chunk),
+            "llama": dict(LLAMA_3_2_1B, vocab_size=vocab, hidden_size=width, intermediate_size=ff, num_hidden_layers=layers,
+                          num_attention_heads=heads, num_key_value_heads=kv_heads, head_dim=64),
+        }
+        for design, raw in shapes.items():
+            if args.design_only and design != args.design_only:
+                continue
+            engine, cfg = make_engine(raw, args.dtype, 64, args.context, args.block_size, budget=8192,
+                                      decode_steps=args.decode_steps)
+            got = {}
+            for n in (2048, 8192):
+                t = prefill_run(engine, cfg, n, repeats=2)
+                got[f"prefill{n}_tok_s"], got[f"prefill{n}_ms"] = round(n / t, 1), round(t * 1e3, 3)
+            for b in (1, 8, 64):
+                tok_s, ms, _ = decode_run(engine, cfg, b, args.context, min(args.steps, 32), min(args.warmup, 4),
+                                          args.decode_steps)
+                got[f"decode_b{b}_tok_s"], got[f"decode_b{b}_ms"] = round(tok_s, 1), round(ms, 4)
+            out[f"{design}_{name}"] = got
+            del engine
+            gc.collect()
+            torch.cuda.empty_cache()
+    return out
+
+
 def other_shapes(args, short, itemsize):
     """The baseline's other workloads, each on a model of its own sizes: flat entries for ``points``."""
     import gc
@@ -327,6 +384,12 @@ def main() -> int:
                     help="prompt length of --only-prefill (the line of the default run always has 2,048)")
     ap.add_argument("--portion", type=int, default=None,
                     help="with --only-prefill: the prompt runs in steps of at most this many tokens")
+    ap.add_argument("--design", default=None, choices=["makodra"],
+                    help="instead of the default run: prefill (2,048 and 8,192 tokens) and decode (batch 1, 8, 64 at "
+                         "--context) of this design beside the Llama decoder at equal sizes, random weights")
+    ap.add_argument("--design-sizes", default="1024,2048", help="widths of --design, of " + ", ".join(DESIGN_SIZES))
+    ap.add_argument("--design-only", default=None, choices=["makodra", "llama"],
+                    help="with --design: measure this one of the pair alone (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on one GPU)")
@@ -347,6 +410,15 @@ def main() -> int:
         raw["num_hidden_layers"] = args.layers
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     itemsize = 2 if short == "bf16" else 4
+    if args.design:
+        print(json.dumps({
+            "metric": f"{args.design} beside llama at equal sizes: prefill and decode tok/s", "unit": "tok/s", "n_gpus": 1,
+            "dtype": short, "data": "synthetic: random token ids, random-init weights N(0, 0.02)",
+            "config": {"context": args.context, "kv_block_size": args.block_size, "sizes": {
+                n: dict(zip(("width", "heads_of_64", "kv_heads", "ff", "layers", "vocab", "chunk"), DESIGN_SIZES[n]))
+                for n in args.design_sizes.split(",")}},
+            "results": design_compare(args)}))
+        return 0
     if args.serving:
         got, cfg = serving_run(raw, args.dtype, args.serving, args.budget, min(args.decode_steps, 8))
         print(json.dumps({

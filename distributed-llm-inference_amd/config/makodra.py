@@ -88,6 +88,19 @@ class MakodraConfig:
 
     architecture = "Makodra"
 
+    # the names under which the engine's tools ask any configuration for its common sizes
+    @property
+    def vocab_size(self) -> int:
+        return self.vocab
+
+    @property
+    def hidden_size(self) -> int:
+        return self.width
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
     @classmethod
     def from_dict(cls, raw: Mapping[str, Any]) -> "MakodraConfig":
         layers = _need(raw, "layers", "")

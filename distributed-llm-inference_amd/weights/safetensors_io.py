@@ -184,11 +184,12 @@ def write_safetensors(
         if tag not in _NUMPY_OF_TAG:
             raise SafetensorsFormatError(f"unknown dtype tag {tag!r} for {name!r}")
         dt = _NUMPY_OF_TAG[tag]
+        shape = list(np.shape(arr))  # (a scalar stays a scalar: ascontiguousarray gives it one dimension)
         arr = np.ascontiguousarray(arr)
         if arr.dtype.itemsize != dt.itemsize:
             raise SafetensorsFormatError(f"{name!r}: array of {arr.dtype} cannot be stored as {tag}")
         raw = np.ascontiguousarray(arr.astype(dt, copy=False) if arr.dtype != dt else arr)
-        header[name] = {"dtype": tag, "shape": list(arr.shape), "data_offsets": [offset, offset + raw.nbytes]}
+        header[name] = {"dtype": tag, "shape": shape, "data_offsets": [offset, offset + raw.nbytes]}
         blobs.append(raw)
         offset += raw.nbytes
     text = json.dumps(header, separators=(",", ":")).encode("utf-8")
