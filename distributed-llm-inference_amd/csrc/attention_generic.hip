@@ -21,8 +21,8 @@
 //   value_dim     the size of a value where it differs from a key's;
 //   gate          float32 [tokens][gate_stride]: the result is multiplied by sigmoid(gate) element
 //                 by element (same layout as the output).
-// tile_entry == nullptr: tile t is the single row of entry t (steps of single tokens, whose
-// launches read nothing that the host made from the step's lengths).
+// tile_entry == nullptr: every entry is a single row (steps of single tokens, whose launches read
+// nothing that the host made from the step's lengths); a kernel of its own takes these, below.
 //
 // Page layout: K [pages][kv_heads][page_size][head_dim], V [pages][kv_heads][value_dim][page_size].
 #include "common.h"
@@ -212,6 +212,192 @@ static int launch_generic(const void* q, int64_t q_stride, const void* k_pages, 
   return dli_launch_status();
 }
 
+// ---------------------------------------------------------------------------------------------
+// Steps of single tokens: one workgroup takes one (entry, kv head, group of up to GQ query heads
+// that share it) and its four waves take the blocks of 64 visible keys in turn. In a block, lane j
+// owns key j: it reads the key's row (16 bytes at a time) and makes its GQ scores against the
+// queries in LDS, the changes to the scores are applied, and each head's reference point moves to
+// the block's maximum (one wave reduction a head); the weights then go through LDS and the lanes
+// change roles: lane c owns value column c (+ 64, ...) and adds up the block's 64 keys, whose
+// values lie side by side in a page's row. The four waves' states are merged through LDS at the
+// end. The same arithmetic as the tile kernel, in another order: 32-bit throughout.
+template <typename T> struct Pack16;   // what 16 bytes hold
+template <> struct Pack16<bf16_t> { static constexpr int N = 8; typedef __bf16 type __attribute__((ext_vector_type(8))); };
+template <> struct Pack16<float> { static constexpr int N = 4; typedef float type __attribute__((ext_vector_type(4))); };
+
+template <typename T, int GQ, int VC>
+__global__ __launch_bounds__(256) void attention_scored_decode_kernel(
+    const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
+    T* __restrict__ out, int64_t out_stride, const int* __restrict__ kv_len, const int* __restrict__ block_tables,
+    int table_stride, int q_heads, int kv_heads, int head_dim, int page_size, float scale, int window,
+    ScoreChanges sc) {
+  constexpr int PN = Pack16<T>::N;
+  typedef typename Pack16<T>::type P16;
+  extern __shared__ float lds[];
+  const int value_dim = sc.value_dim;
+  float* qs = lds;                               // [GQ][head_dim]
+  float* ps = qs + GQ * head_dim;                // [4][GQ][64]
+  float* ms = ps + 4 * GQ * 64;                  // [4][GQ] reference points, then [4][GQ] sums
+  float* accs = ms + 8 * GQ;                     // [4][GQ][VC * 64]
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int entry = blockIdx.x, kvh = blockIdx.y;
+  const int group = q_heads / kv_heads;
+  const int h0 = kvh * group + blockIdx.z * GQ;                  // first query head of this workgroup
+  const int nh = min(GQ, kvh * group + group - h0);              // heads that exist
+  const int n_keys = kv_len[entry];
+  const int pos = n_keys - 1;
+  const int* table = block_tables + (int64_t)entry * table_stride;
+
+  for (int idx = tid; idx < GQ * head_dim; idx += 256) {
+    const int h = idx / head_dim, c = idx - h * head_dim;
+    qs[idx] = h < nh ? to_f32(q[(int64_t)entry * q_stride + (int64_t)(h0 + h) * head_dim + c]) * scale : 0.f;
+  }
+  float r1[GQ], r2[GQ], m_run[GQ], l_run[GQ], acc[GQ][VC];
+#pragma unroll
+  for (int h = 0; h < GQ; ++h) {
+    r1[h] = sc.r1 != nullptr && h < nh ? sc.r1[h0 + h] : 0.f;
+    r2[h] = sc.r1 != nullptr && h < nh ? sc.r2[h0 + h] : 0.f;
+    m_run[h] = sc.sink && wave == 0 ? 0.f : -INFINITY;           // the sink is counted once, by wave 0
+    l_run[h] = sc.sink && wave == 0 && lane == 0 ? 1.f : 0.f;    // (sums are kept lane by lane until the end)
+#pragma unroll
+    for (int c = 0; c < VC; ++c) acc[h][c] = 0.f;
+  }
+  int j_begin = 0;
+  if (window > 0) j_begin = max(0, pos - window + 1);
+  if (sc.chunk > 0) j_begin = max(j_begin, pos / sc.chunk * sc.chunk);
+  __syncthreads();
+
+  const bool k_packs = head_dim % PN == 0, v_packs = page_size % PN == 0;
+  for (int j0 = j_begin / 64 * 64 + wave * 64; j0 <= pos; j0 += 256) {
+    const int j = j0 + lane;
+    const bool seen = j >= j_begin && j <= pos;
+    float s[GQ];
+#pragma unroll
+    for (int h = 0; h < GQ; ++h) s[h] = 0.f;
+    if (seen) {
+      const int64_t page = table[j / page_size];
+      const T* kr = k_pages + ((page * kv_heads + kvh) * page_size + j % page_size) * head_dim;
+      if (k_packs) {
+        for (int d = 0; d < head_dim; d += PN) {
+          const P16 kk = *reinterpret_cast<const P16*>(kr + d);
+#pragma unroll
+          for (int e = 0; e < PN; ++e) {
+            const float kf = to_f32((T)kk[e]);
+#pragma unroll
+            for (int h = 0; h < GQ; ++h) s[h] = fmaf(qs[h * head_dim + d + e], kf, s[h]);
+          }
+        }
+      } else {
+        for (int d = 0; d < head_dim; ++d) {
+          const float kf = to_f32(kr[d]);
+#pragma unroll
+          for (int h = 0; h < GQ; ++h) s[h] = fmaf(qs[h * head_dim + d], kf, s[h]);
+        }
+      }
+    }
+    const float dist = (float)(pos - j);
+#pragma unroll
+    for (int h = 0; h < GQ; ++h) {
+      float sh = seen ? s[h] - (sc.r1 != nullptr ? r1[h] * log1pf(r2[h] * dist) : 0.f) : -INFINITY;
+      const float m_new = fmaxf(m_run[h], wave_max(sh));
+      float p = 0.f, alpha = 1.f;
+      if (m_new > -INFINITY) {
+        alpha = expf(m_run[h] - m_new);
+        p = expf(sh - m_new);
+      }
+      l_run[h] = l_run[h] * alpha + p;
+      m_run[h] = m_new;
+#pragma unroll
+      for (int c = 0; c < VC; ++c) acc[h][c] *= alpha;
+      ps[(wave * GQ + h) * 64 + lane] = p;
+    }
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    // lanes are value columns now
+    const int last = min(63, pos - j0);
+    const int first = max(0, j_begin - j0);
+#pragma unroll
+    for (int c = 0; c < VC; ++c) {
+      const int col = lane + 64 * c;
+      if (col < value_dim) {
+        int jj = first;
+        while (jj <= last) {
+          const int jk = j0 + jj;
+          const int64_t page = table[jk / page_size];
+          const int off = jk % page_size;
+          const T* vr = v_pages + ((page * kv_heads + kvh) * value_dim + col) * page_size + off;
+          if (v_packs && off % PN == 0 && jj + PN - 1 <= last) {
+            const P16 vv = *reinterpret_cast<const P16*>(vr);
+#pragma unroll
+            for (int e = 0; e < PN; ++e) {
+              const float vf = to_f32((T)vv[e]);
+#pragma unroll
+              for (int h = 0; h < GQ; ++h) acc[h][c] = fmaf(ps[(wave * GQ + h) * 64 + jj + e], vf, acc[h][c]);
+            }
+            jj += PN;
+          } else {
+            const float vf = to_f32(vr[0]);
+#pragma unroll
+            for (int h = 0; h < GQ; ++h) acc[h][c] = fmaf(ps[(wave * GQ + h) * 64 + jj], vf, acc[h][c]);
+            jj += 1;
+          }
+        }
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+
+  // the four waves' states meet: reference points and sums first, then the accumulators
+#pragma unroll
+  for (int h = 0; h < GQ; ++h) {
+    const float l = wave_sum(l_run[h]);
+    if (lane == 0) {
+      ms[wave * GQ + h] = m_run[h];
+      ms[4 * GQ + wave * GQ + h] = l;
+    }
+#pragma unroll
+    for (int c = 0; c < VC; ++c) accs[((wave * GQ + h) * VC + c) * 64 + lane] = acc[h][c];
+  }
+  __syncthreads();
+  for (int idx = tid; idx < nh * value_dim; idx += 256) {
+    const int h = idx / value_dim, col = idx - h * value_dim;
+    float m = -INFINITY;
+    for (int w = 0; w < 4; ++w) m = fmaxf(m, ms[w * GQ + h]);
+    float l = 0.f, o = 0.f;
+    for (int w = 0; w < 4; ++w) {
+      const float mw = ms[w * GQ + h];
+      if (mw > -INFINITY) {
+        const float f = expf(mw - m);
+        l += ms[4 * GQ + w * GQ + h] * f;
+        o += accs[((w * GQ + h) * VC + col / 64) * 64 + col % 64] * f;
+      }
+    }
+    float y = l > 0.f ? o / l : 0.f;
+    const int64_t at = (int64_t)(h0 + h) * value_dim + col;
+    if (sc.gate != nullptr) y *= 1.f / (1.f + expf(-sc.gate[(int64_t)entry * sc.gate_stride + at]));
+    out[(int64_t)entry * out_stride + at] = from_f32<T>(y);
+  }
+}
+
+template <typename T, int GQ>
+static int launch_scored_decode(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages, void* out,
+                                int64_t out_stride, const int* kv_len, const int* block_tables, int table_stride,
+                                int entries, int q_heads, int kv_heads, int head_dim, int page_size, float scale,
+                                int window, ScoreChanges sc, hipStream_t stream) {
+  const int group = q_heads / kv_heads, vc = (sc.value_dim + 63) / 64;
+  const dim3 grid(entries, kv_heads, (group + GQ - 1) / GQ);
+#define DECODE_LAUNCH(VC)                                                                                   \
+  {                                                                                                         \
+    const size_t bytes = sizeof(float) * ((size_t)GQ * head_dim + 4 * GQ * 64 + 8 * GQ + 4 * GQ * VC * 64); \
+    attention_scored_decode_kernel<T, GQ, VC><<<grid, 256, bytes, stream>>>(                                \
+        (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, kv_len,           \
+        block_tables, table_stride, q_heads, kv_heads, head_dim, page_size, scale, window, sc);             \
+  }
+  if (vc <= 1) DECODE_LAUNCH(1) else if (vc == 2) DECODE_LAUNCH(2) else DECODE_LAUNCH(4)
+#undef DECODE_LAUNCH
+  return dli_launch_status();
+}
+
 // Queries per tile for a head_dim (the larger of the key's and the value's size): the host builds
 // its tile list with this.
 extern "C" int dli_attention_generic_tile_rows(int head_dim) {
@@ -237,6 +423,22 @@ extern "C" int dli_attention_scored(const void* q, int64_t q_stride, const void*
       (tile_entry == nullptr) != (tile_q0 == nullptr))
     return DLI_ERR_ARGUMENT;
   const ScoreChanges sc = {chunk, sink, r1, r2, value_dim, gate, gate_stride};
+  if (tile_entry == nullptr) {
+    // every entry is one row: the kernel whose lanes own keys, then value columns
+    const int group = q_heads / kv_heads;
+#define DECODE_ARGS                                                                                      \
+  q, q_stride, k_pages, v_pages, out, out_stride, kv_len, block_tables, table_stride, tiles, q_heads,   \
+      kv_heads, head_dim, page_size, scale, window, sc, stream
+    if (is_bf16) {
+      if (group == 1) return launch_scored_decode<bf16_t, 1>(DECODE_ARGS);
+      if (group <= 4) return launch_scored_decode<bf16_t, 4>(DECODE_ARGS);
+      return launch_scored_decode<bf16_t, 8>(DECODE_ARGS);
+    }
+    if (group == 1) return launch_scored_decode<float, 1>(DECODE_ARGS);
+    if (group <= 4) return launch_scored_decode<float, 4>(DECODE_ARGS);
+    return launch_scored_decode<float, 8>(DECODE_ARGS);
+#undef DECODE_ARGS
+  }
 #define GENERIC_ARGS                                                                              \
   q, q_stride, k_pages, v_pages, out, out_stride, q_start, kv_len, block_tables, table_stride,   \
       tile_entry, tile_q0, tiles, q_heads, kv_heads, head_dim, page_size, scale, window, sc, stream

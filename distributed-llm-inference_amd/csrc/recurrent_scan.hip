@@ -9,13 +9,15 @@
 // sigmoid(g_pre) (RULE_DELTA) or silu(g_pre) (RULE_BONUS); the result is written in the type of
 // the product that reads it. Everything here is 32-bit arithmetic on 32-bit inputs.
 //
-// One workgroup takes one (entry, head) and walks the entry's tokens in order. Thread
-// (v, part) of D * PARTS threads keeps the D / PARTS state values S[part's keys][v] in registers:
-// a column of S never leaves its PARTS neighbouring lanes, whose partial dot products meet in two
-// lane swaps. The per-token vectors of up to TB tokens are staged in LDS at once (loads and
-// transcendentals of a batch in parallel, the chain over tokens reads LDS only), and the batch's
-// outputs are normalised and gated together afterwards. The sums of a token do not depend on
-// where a step cut the request: the state is the only thing carried, and it is carried exactly.
+// One wave takes one (entry, head, slice of 16 value columns) and walks the entry's tokens in
+// order; waves never wait for each other. Lane (v, part) keeps the D / 4 state values
+// S[part's keys][v] in registers: a column of S never leaves its four neighbouring lanes, whose
+// partial dot products meet in two DPP swaps inside a quad. The per-token vectors of 16 tokens (8 for heads above 64)
+// are staged in LDS at once (the loads of the next batch are in flight while the chain over this
+// batch's tokens runs, and the chain itself reads LDS and registers only). o goes out in 32-bit;
+// a second kernel normalises each head's o and applies the gate (it needs all of a head's
+// columns, which lie in several waves). The sums of a token do not depend on where a step cut the
+// request: the state is the only thing carried, and it is carried exactly.
 //
 // State slot layout: [heads][D (value)][D (key)] floats at `state + slot * state_stride`.
 // A request whose first row of the step has position 0 starts from a zero state.
@@ -35,121 +37,160 @@ struct ScanArgs {
   float eps;
   float* state; int64_t state_stride;
   const int* q_start; const int* positions; const int* state_slots;
+  float* o_raw; int64_t o_stride;                    // the recurrence's own output, before norm and gate
   void* out; int64_t out_stride;
   int heads;
 };
 
-template <typename T, int NK, int RULE>
-__global__ __launch_bounds__(NK * 16) void recurrent_scan_kernel(ScanArgs p) {
-  constexpr int PARTS = 4, D = NK * PARTS, TB = 8, THREADS = D * PARTS;
-  __shared__ float sr[TB][D], sk[TB][D], sv[TB][D], sw[TB][D], sa[TB][D], so[TB][D];
-  __shared__ float knorm[TB], onorm[TB];
-  const int tid = threadIdx.x, vcol = tid / PARTS, part = tid % PARTS;
-  const int lane = tid % DLI_WAVE, wave = tid / DLI_WAVE;
-  constexpr int WAVES = THREADS / DLI_WAVE;  // whole waves: they make the sums over a head (THREADS >= 64)
-  const int entry = blockIdx.x, head = blockIdx.y;
+// Sum over the four lanes of a quad (every lane gets it), by two DPP quad permutes.
+__device__ __forceinline__ float quad_sum(float x) {
+  x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, false));
+  x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, false));
+  return x;
+}
+
+template <int NK, int RULE>
+__global__ __launch_bounds__(64) void recurrent_scan_kernel(ScanArgs p) {
+  constexpr int D = NK * 4, TB = D > 64 ? 8 : 16, PER = TB * D / 64;  // PER: what a lane stages per vector and batch
+  __shared__ float sk[TB * D], sw[TB * D], sa[RULE == RULE_DELTA ? TB * D : 1], sr[TB * D];
+  const int lane = threadIdx.x, vloc = lane >> 2, part = lane & 3;
+  const int entry = blockIdx.x, head = blockIdx.y, col = blockIdx.z * 16 + vloc;
+  const bool live = col < D;
+  const int ccol = live ? col : D - 1;
   const int row0 = p.q_start[entry], n_rows = p.q_start[entry + 1] - row0;
   if (n_rows <= 0) return;
   const int64_t col0 = (int64_t)head * D;
-  float* st = p.state + (int64_t)p.state_slots[entry] * p.state_stride + ((int64_t)head * D + vcol) * D + part * NK;
-  float s[NK];
-  if (p.positions[row0] == 0) {
+  float* st = p.state + (int64_t)p.state_slots[entry] * p.state_stride + ((int64_t)head * D + ccol) * D + part * NK;
+  float s[NK], bon[NK];
+  const bool fresh = p.positions[row0] == 0;
 #pragma unroll
-    for (int i = 0; i < NK; ++i) s[i] = 0.f;
-  } else {
-#pragma unroll
-    for (int i = 0; i < NK; ++i) s[i] = st[i];
+  for (int i = 0; i < NK; ++i) {
+    s[i] = (fresh || !live) ? 0.f : st[i];
+    bon[i] = RULE == RULE_BONUS ? p.bonus[col0 + part * NK + i] : 0.f;
   }
 
+  float pk[PER], pw[PER], pa[PER], pr[PER], pv[TB];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int m = 0; m < PER; ++m) {
+      const int e = lane + 64 * m, t = e / D, c = e - t * D;
+      const int64_t row = row0 + min(t0 + t, n_rows - 1);
+      pk[m] = p.k[row * p.k_stride + col0 + c];
+      pr[m] = p.r[row * p.r_stride + col0 + c];
+      pw[m] = p.w_pre[row * p.w_stride + col0 + c];
+      if (RULE == RULE_DELTA) pa[m] = p.a_pre[row * p.a_stride + col0 + c] + p.a_bias[col0 + c];
+    }
+#pragma unroll
+    for (int t = 0; t < TB; ++t) pv[t] = p.v[(int64_t)(row0 + min(t0 + t, n_rows - 1)) * p.v_stride + col0 + ccol];
+  };
+  fetch(0);
   for (int t0 = 0; t0 < n_rows; t0 += TB) {
+    float vv[TB];
+#pragma unroll
+    for (int m = 0; m < PER; ++m) {
+      const int e = lane + 64 * m;
+      sk[e] = pk[m];
+      sr[e] = pr[m];
+      if (RULE == RULE_DELTA) {
+        sw[e] = expf(-0.6065306597126334f / (1.f + expf(-pw[m])));
+        sa[e] = 1.f / (1.f + expf(-pa[m]));
+      } else {
+        sw[e] = expf(-expf(pw[m]));
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < TB; ++t) vv[t] = live ? pv[t] : 0.f;
+    if (t0 + TB < n_rows) fetch(t0 + TB);  // on their way while the chain below runs
+    __syncthreads();                       // (one wave: orders its LDS writes before its reads)
     const int nb = min(TB, n_rows - t0);
-    __syncthreads();  // the batch before is read out
-    for (int idx = tid; idx < nb * D; idx += THREADS) {
-      const int t = idx / D, c = idx - t * D;
-      const int64_t row = row0 + t0 + t;
-      sr[t][c] = p.r[row * p.r_stride + col0 + c];
-      sk[t][c] = p.k[row * p.k_stride + col0 + c];
-      sv[t][c] = p.v[row * p.v_stride + col0 + c];
-      const float wp = p.w_pre[row * p.w_stride + col0 + c];
-      if (RULE == RULE_DELTA) {
-        sw[t][c] = expf(-0.6065306597126334f / (1.f + expf(-wp)));
-        sa[t][c] = 1.f / (1.f + expf(-(p.a_pre[row * p.a_stride + col0 + c] + p.a_bias[col0 + c])));
-      } else {
-        sw[t][c] = expf(-expf(wp));
-        sa[t][c] = p.bonus[col0 + c];
-      }
-    }
-    __syncthreads();
-    if (RULE == RULE_DELTA) {
-      for (int t = wave; t < nb && wave < WAVES; t += WAVES) {
-        float ss = 0.f;
-        for (int c = lane; c < D; c += DLI_WAVE) ss += sk[t][c] * sk[t][c];
-        ss = wave_sum(ss);
-        if (lane == 0) knorm[t] = 1.f / sqrtf(ss + 1e-6f);
-      }
-      __syncthreads();
-    }
-    for (int t = 0; t < nb; ++t) {
-      const float vv = sv[t][vcol];
-      float o = 0.f;
-      if (RULE == RULE_DELTA) {
-        const float kn = knorm[t];
-        float us = 0.f;
 #pragma unroll
-        for (int i = 0; i < NK; ++i) us = fmaf(sk[t][part * NK + i] * kn, s[i], us);
-        us += __shfl_xor(us, 1, DLI_WAVE);
-        us += __shfl_xor(us, 2, DLI_WAVE);
+    for (int t = 0; t < TB; ++t) {
+      if (t < nb) {
+        const float* kt = sk + t * D + part * NK;
+        const float* wt = sw + t * D + part * NK;
+        const float* rt = sr + t * D + part * NK;
+        float o0 = 0.f, o1 = 0.f;
+        if (RULE == RULE_DELTA) {
+          const float* at = sa + t * D + part * NK;
+          float ks0 = 0.f, ks1 = 0.f, kk = 0.f;
 #pragma unroll
-        for (int i = 0; i < NK; ++i) {
-          const int c = part * NK + i;
-          const float kk = sk[t][c], u = kk * kn;
-          s[i] = sw[t][c] * s[i] - (sa[t][c] * u) * us + kk * vv;
-          o = fmaf(s[i], sr[t][c], o);
+          for (int i = 0; i < NK; i += 2) {
+            ks0 = fmaf(kt[i], s[i], ks0);
+            ks1 = fmaf(kt[i + 1], s[i + 1], ks1);
+            kk = fmaf(kt[i], kt[i], kk);
+            kk = fmaf(kt[i + 1], kt[i + 1], kk);
+          }
+          const float kn = 1.f / sqrtf(quad_sum(kk) + 1e-6f);
+          const float us = quad_sum(ks0 + ks1) * kn;       // u^T S for this column, u = k * kn
+#pragma unroll
+          for (int i = 0; i < NK; i += 2) {
+            s[i] = wt[i] * s[i] - (at[i] * (kt[i] * kn)) * us + kt[i] * vv[t];
+            s[i + 1] = wt[i + 1] * s[i + 1] - (at[i + 1] * (kt[i + 1] * kn)) * us + kt[i + 1] * vv[t];
+            o0 = fmaf(s[i], rt[i], o0);
+            o1 = fmaf(s[i + 1], rt[i + 1], o1);
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < NK; i += 2) {
+            const float kv0 = kt[i] * vv[t], kv1 = kt[i + 1] * vv[t];
+            o0 = fmaf(s[i] + bon[i] * kv0, rt[i], o0);
+            o1 = fmaf(s[i + 1] + bon[i + 1] * kv1, rt[i + 1], o1);
+            s[i] = wt[i] * s[i] + kv0;
+            s[i + 1] = wt[i + 1] * s[i + 1] + kv1;
+          }
         }
-      } else {
-#pragma unroll
-        for (int i = 0; i < NK; ++i) {
-          const int c = part * NK + i;
-          const float kv = sk[t][c] * vv;
-          o = fmaf(s[i] + sa[t][c] * kv, sr[t][c], o);
-          s[i] = sw[t][c] * s[i] + kv;
-        }
+        const float o = quad_sum(o0 + o1);
+        if (part == 0 && live) p.o_raw[(int64_t)(row0 + t0 + t) * p.o_stride + col0 + col] = o;
       }
-      o += __shfl_xor(o, 1, DLI_WAVE);
-      o += __shfl_xor(o, 2, DLI_WAVE);
-      if (part == 0) so[t][vcol] = o;
     }
-    __syncthreads();
-    for (int t = wave; t < nb && wave < WAVES; t += WAVES) {
-      float ss = 0.f;
-      for (int c = lane; c < D; c += DLI_WAVE) ss += so[t][c] * so[t][c];
-      ss = wave_sum(ss);
-      if (lane == 0) onorm[t] = 1.f / sqrtf(ss / (float)D + p.eps);
-    }
-    __syncthreads();
-    for (int idx = tid; idx < nb * D; idx += THREADS) {
-      const int t = idx / D, c = idx - t * D;
-      const int64_t row = row0 + t0 + t;
-      const float g = p.g_pre[row * p.g_stride + col0 + c];
-      const float gate = RULE == RULE_DELTA ? 1.f / (1.f + expf(-g)) : g / (1.f + expf(-g));
-      ((T*)p.out)[row * p.out_stride + col0 + c] = from_f32<T>(so[t][c] * onorm[t] * p.norm_w[col0 + c] * gate);
-    }
+    __syncthreads();  // the chain has read this batch before the next one is written
   }
+  if (live) {
 #pragma unroll
-  for (int i = 0; i < NK; ++i) st[i] = s[i];
+    for (int i = 0; i < NK; ++i) st[i] = s[i];
+  }
 }
 
+// out = o / sqrt(mean_head(o^2) + eps) * norm_w * gate(g_pre), head by head: one workgroup a row,
+// its waves take the heads in turn.
 template <typename T, int RULE>
-static int launch_scan(const ScanArgs& p, int entries, int dim, hipStream_t stream) {
-  const dim3 grid(entries, p.heads);
+__global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, int64_t o_stride,
+                                                             const float* __restrict__ g_pre, int64_t g_stride,
+                                                             const float* __restrict__ norm_w, float eps,
+                                                             T* __restrict__ out, int64_t out_stride, int heads, int dim) {
+  const int64_t row = blockIdx.x;
+  const int lane = threadIdx.x % DLI_WAVE, wave = threadIdx.x / DLI_WAVE;
+  for (int h = wave; h < heads; h += 4) {
+    const float* oh = o + row * o_stride + (int64_t)h * dim;
+    float ss = 0.f;
+    for (int c = lane; c < dim; c += DLI_WAVE) ss += oh[c] * oh[c];
+    const float r = 1.f / sqrtf(wave_sum(ss) / (float)dim + eps);
+    for (int c = lane; c < dim; c += DLI_WAVE) {
+      const float g = g_pre[row * g_stride + (int64_t)h * dim + c];
+      const float gate = RULE == RULE_DELTA ? 1.f / (1.f + expf(-g)) : g / (1.f + expf(-g));
+      out[row * out_stride + (int64_t)h * dim + c] = from_f32<T>(oh[c] * r * norm_w[(int64_t)h * dim + c] * gate);
+    }
+  }
+}
+
+template <int RULE>
+static int launch_scan(const ScanArgs& p, int entries, int rows, int dim, int out_is_bf16, hipStream_t stream) {
+  const dim3 grid(entries, p.heads, (dim + 15) / 16);
 #define SCAN_CASE(NK) \
-  case NK: recurrent_scan_kernel<T, NK, RULE><<<grid, NK * 16, 0, stream>>>(p); break;
+  case NK: recurrent_scan_kernel<NK, RULE><<<grid, 64, 0, stream>>>(p); break;
   switch (dim / 4) {
     SCAN_CASE(4) SCAN_CASE(6) SCAN_CASE(8) SCAN_CASE(10) SCAN_CASE(12) SCAN_CASE(14) SCAN_CASE(16)
     SCAN_CASE(20) SCAN_CASE(24) SCAN_CASE(28) SCAN_CASE(32)
     default: return DLI_ERR_ARGUMENT;
   }
 #undef SCAN_CASE
+  if (dli_launch_status() != DLI_OK) return DLI_ERR_LAUNCH;
+  if (out_is_bf16)
+    head_norm_gate_kernel<bf16_t, RULE><<<rows, 256, 0, stream>>>(p.o_raw, p.o_stride, p.g_pre, p.g_stride, p.norm_w, p.eps,
+                                                                  (bf16_t*)p.out, p.out_stride, p.heads, dim);
+  else
+    head_norm_gate_kernel<float, RULE><<<rows, 256, 0, stream>>>(p.o_raw, p.o_stride, p.g_pre, p.g_stride, p.norm_w, p.eps,
+                                                                 (float*)p.out, p.out_stride, p.heads, dim);
   return dli_launch_status();
 }
 
@@ -164,9 +205,10 @@ extern "C" int dli_recurrent_scan(const float* r, int64_t r_stride, const float*
                                   int64_t a_stride, const float* a_bias, const float* g_pre, int64_t g_stride,
                                   const float* bonus, const float* norm_w, float eps, float* state,
                                   int64_t state_stride, const int* q_start, const int* positions,
-                                  const int* state_slots, void* out, int64_t out_stride, int entries, int heads,
-                                  int dim, int rule, int out_is_bf16, hipStream_t stream) {
-  if (entries <= 0) return DLI_OK;
+                                  const int* state_slots, float* o_raw, int64_t o_stride, void* out,
+                                  int64_t out_stride, int entries, int rows, int heads, int dim, int rule,
+                                  int out_is_bf16, hipStream_t stream) {
+  if (entries <= 0 || rows <= 0) return DLI_OK;
   if (!dli_recurrent_scan_supports(dim) || heads <= 0 || heads > 65535 || (rule != RULE_DELTA && rule != RULE_BONUS) ||
       state_stride < (int64_t)heads * dim * dim || (rule == RULE_DELTA && (a_pre == nullptr || a_bias == nullptr)) ||
       (rule == RULE_BONUS && bonus == nullptr))
@@ -177,10 +219,9 @@ extern "C" int dli_recurrent_scan(const float* r, int64_t r_stride, const float*
   p.a_stride = a_stride; p.g_stride = g_stride;
   p.bonus = bonus; p.norm_w = norm_w; p.eps = eps; p.state = state; p.state_stride = state_stride;
   p.q_start = q_start; p.positions = positions; p.state_slots = state_slots; p.out = out; p.out_stride = out_stride;
+  p.o_raw = o_raw; p.o_stride = o_stride;
   p.heads = heads;
-  if (rule == RULE_DELTA)
-    return out_is_bf16 ? launch_scan<bf16_t, RULE_DELTA>(p, entries, dim, stream)
-                       : launch_scan<float, RULE_DELTA>(p, entries, dim, stream);
-  return out_is_bf16 ? launch_scan<bf16_t, RULE_BONUS>(p, entries, dim, stream)
-                     : launch_scan<float, RULE_BONUS>(p, entries, dim, stream);
+  if (o_raw == nullptr || o_stride < (int64_t)heads * dim) return DLI_ERR_ARGUMENT;
+  return rule == RULE_DELTA ? launch_scan<RULE_DELTA>(p, entries, rows, dim, out_is_bf16, stream)
+                            : launch_scan<RULE_BONUS>(p, entries, rows, dim, out_is_bf16, stream);
 }

@@ -11,7 +11,7 @@
 //   token_shift        S mixes of each row with the row before it, x + (prev - x) * mu_s; the row
 //                      before a step's first row comes from the request's state, which then
 //                      receives the step's last row
-//   lowrank_out        y = bias + W2 act(t): the second half of a low-rank projection, 32-bit
+//   lowrank_out        y = bias + W2 act(t): the second half of a low-rank projection, 32-bit (W2 given transposed)
 //   qk_unit_cache      per-head unit RMS of q and k, value mixing, cache write
 #include "common.h"
 
@@ -106,8 +106,9 @@ __global__ void token_shift_kernel(const float* __restrict__ x, const float* __r
   }
 }
 
-// act: 0 none, 1 tanh. t is [rows][t_stride] (rank values a row), w2 [features][rank], out [rows][features].
-__global__ void lowrank_out_kernel(const float* __restrict__ t, int64_t t_stride, const float* __restrict__ w2,
+// act: 0 none, 1 tanh. t is [rows][t_stride] (rank values a row), w2t [rank][features] (the matrix
+// transposed, so that neighbouring threads read neighbouring weights), out [rows][features].
+__global__ void lowrank_out_kernel(const float* __restrict__ t, int64_t t_stride, const float* __restrict__ w2t,
                                    const float* __restrict__ bias, float* __restrict__ out, int features, int rank,
                                    int act) {
   extern __shared__ float ts[];
@@ -119,7 +120,7 @@ __global__ void lowrank_out_kernel(const float* __restrict__ t, int64_t t_stride
   __syncthreads();
   for (int c = threadIdx.x; c < features; c += blockDim.x) {
     float s = 0.f;
-    for (int j = 0; j < rank; ++j) s = fmaf(ts[j], w2[(int64_t)c * rank + j], s);
+    for (int j = 0; j < rank; ++j) s = fmaf(ts[j], w2t[(int64_t)j * features + c], s);
     out[row * features + c] = s + (bias != nullptr ? bias[c] : 0.f);
   }
 }
@@ -237,11 +238,11 @@ int dli_token_shift(const float* x, const float* mu, int mixes, float* state, in
   return dli_launch_status();
 }
 
-int dli_lowrank_out(const float* t, int64_t t_stride, const float* w2, const float* bias, float* out, int rows,
+int dli_lowrank_out(const float* t, int64_t t_stride, const float* w2t, const float* bias, float* out, int rows,
                     int features, int rank, int act, hipStream_t stream) {
   if (rows <= 0) return DLI_OK;
   if (features <= 0 || rank <= 0 || rank > 8192 || t_stride < rank || act < 0 || act > 1) return DLI_ERR_ARGUMENT;
-  lowrank_out_kernel<<<rows, 256, rank * sizeof(float), stream>>>(t, t_stride, w2, bias, out, features, rank, act);
+  lowrank_out_kernel<<<rows, 256, rank * sizeof(float), stream>>>(t, t_stride, w2t, bias, out, features, rank, act);
   return dli_launch_status();
 }
 

@@ -112,8 +112,8 @@ _SIGNATURES = {
                           _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "dli_recurrent_scan_supports": [_c_int],
     "dli_recurrent_scan": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr,
-                           _c_i64, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64,
-                           _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+                           _c_i64, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr,
+                           _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
 }
 
 _lib: Optional[ctypes.CDLL] = None
@@ -1408,21 +1408,22 @@ def token_shift(x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, q_start:
                                      _is_bf16(out.dtype), _stream()), "token_shift")
 
 
-def lowrank_out(t: torch.Tensor, w2: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+def lowrank_out(t: torch.Tensor, w2t: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                 act: str = "tanh") -> None:
-    """``out = act(t) @ w2.T + bias`` in 32-bit: ``t`` float32 ``[n, rank]`` (rows contiguous, any row
-    stride), ``w2`` float32 ``[features, rank]``; ``act`` ``"tanh"`` or ``"none"``."""
+    """``out = act(t) @ w2t + bias`` in 32-bit: ``t`` float32 ``[n, rank]`` (rows contiguous, any row
+    stride), ``w2t`` float32 ``[rank, features]`` (the projection's second matrix transposed);
+    ``act`` ``"tanh"`` or ``"none"``."""
     _f32_rows(t, "t")
-    _dense(w2, "w2", torch.float32, 2)
+    _dense(w2t, "w2t", torch.float32, 2)
     _dense(out, "out", torch.float32, 2)
     _require(act in ("tanh", "none"), "act must be 'tanh' or 'none'")
     n, rank = t.shape
-    feats = w2.shape[0]
-    _require(w2.shape[1] == rank and out.shape == (n, feats), "t, w2 and out disagree on the sizes")
+    feats = w2t.shape[1]
+    _require(w2t.shape[0] == rank and out.shape == (n, feats), "t, w2t and out disagree on the sizes")
     if bias is not None:
         _dense(bias, "bias", torch.float32, 1)
-        _require(bias.shape[0] == feats, "bias length differs from rows of w2")
-    _check(library().dli_lowrank_out(_ptr(t), t.stride(0), _ptr(w2), _ptr(bias), _ptr(out), n, feats, rank,
+        _require(bias.shape[0] == feats, "bias length differs from the features")
+    _check(library().dli_lowrank_out(_ptr(t), t.stride(0), _ptr(w2t), _ptr(bias), _ptr(out), n, feats, rank,
                                      1 if act == "tanh" else 0, _stream()), "lowrank_out")
 
 
@@ -1558,8 +1559,9 @@ def recurrent_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, w_pre: tor
         _dense(bonus, "bonus", torch.float32)
         _require(bonus.numel() == width, "bonus must hold heads*dim values")
     sa = a_pre.stride(0) if a_pre is not None else 0
+    o_raw = torch.empty(n, width, device=out.device, dtype=torch.float32)  # the recurrence's output before norm and gate
     _check(library().dli_recurrent_scan(
         _ptr(r), r.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(w_pre), w_pre.stride(0), _ptr(a_pre), sa,
         _ptr(a_bias), _ptr(g_pre), g_pre.stride(0), _ptr(bonus), _ptr(norm_w), float(eps), _ptr(state), state.stride(0),
-        _ptr(q_start), _ptr(positions), _ptr(state_slots), _ptr(out), out.stride(0), entries, heads, dim, int(rule),
-        _is_bf16(out.dtype), _stream()), "recurrent_scan")
+        _ptr(q_start), _ptr(positions), _ptr(state_slots), _ptr(o_raw), o_raw.stride(0), _ptr(out), out.stride(0), entries,
+        n, heads, dim, int(rule), _is_bf16(out.dtype), _stream()), "recurrent_scan")

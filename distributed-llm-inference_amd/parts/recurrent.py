@@ -40,7 +40,7 @@ class _MatrixStateMixer(Mixer):
         self.hidden_size, self.num_heads, self.head_dim = hidden_size, num_heads, head_dim
         self.norm_eps, self.decay_rank = float(norm_eps), decay_rank
         self.width = num_heads * head_dim
-        self.w2 = self.w0 = self.norm_w = self.w_o = None
+        self.w2t = self.w0 = self.norm_w = self.w_o = None
 
     def _shared_specs(self) -> dict[str, WeightSpec]:
         h, c = self.hidden_size, self.width
@@ -54,7 +54,7 @@ class _MatrixStateMixer(Mixer):
     def _load_shared(self, tensors: Mapping[str, torch.Tensor]) -> None:
         if tensors["w1"].shape[0] != tensors["w2"].shape[1]:
             raise ValueError(f"{self.prefix}w1 and {self.prefix}w2 disagree on the rank of the decay's projection")
-        self.w2, self.w0 = tensors["w2"].contiguous(), tensors["w0"]
+        self.w2t, self.w0 = tensors["w2"].t().contiguous(), tensors["w0"]  # [rank, features]: the kernel's order
         self.norm_w, self.w_o = tensors["norm"], tensors["o"]
 
     def graph_capturable(self, page_size: int) -> bool:
@@ -99,7 +99,7 @@ class GeneralDelta(_MatrixStateMixer):
         proj = linear_f32(self.rt, as_operand(self.rt, x), self.w_in)
         r, k, v, g, a = (proj[:, i * c:(i + 1) * c] for i in range(5))
         w_pre = torch.empty(n, c, device=self.rt.device, dtype=torch.float32)
-        ops.lowrank_out(proj[:, 5 * c:5 * c + self.rank], self.w2, self.w0, w_pre, act="tanh")
+        ops.lowrank_out(proj[:, 5 * c:5 * c + self.rank], self.w2t, self.w0, w_pre, act="tanh")
         out = self.rt.empty(n, c)
         ops.recurrent_scan(r, k, v, w_pre, g, self.norm_w, self.norm_eps, state, ctx.q_start, ctx.positions,
                            ctx.state_slots, out, self.num_heads, self.head_dim, self.rule, a_pre=a, a_bias=self.a_bias)
@@ -144,13 +144,13 @@ class WKV(_MatrixStateMixer):
         n, c, h = x.shape[0], self.width, self.hidden_size
         mixes = self.rt.empty(len(self.MIXES), n, h)
         ops.token_shift(x, self.mu, state, ctx.q_start, ctx.positions, ctx.state_slots, mixes)
-        proj = torch.empty(n, 4 * c + self.rank, device=self.rt.device, dtype=torch.float32)
+        proj = torch.empty(n, 4 * c + -(-self.rank // 8) * 8, device=self.rt.device, dtype=torch.float32)
         for i, name in enumerate(("r", "k", "v", "g")):
             linear_f32(self.rt, mixes[i], self.w[name], out=proj[:, i * c:(i + 1) * c])
-        linear_f32(self.rt, mixes[4], self.w1, out=proj[:, 4 * c:])
+        linear_f32(self.rt, mixes[4], self.w1, out=proj[:, 4 * c:4 * c + self.rank])
         r, k, v, g = (proj[:, i * c:(i + 1) * c] for i in range(4))
         w_pre = torch.empty(n, c, device=self.rt.device, dtype=torch.float32)
-        ops.lowrank_out(proj[:, 4 * c:], self.w2, self.w0, w_pre, act="tanh")
+        ops.lowrank_out(proj[:, 4 * c:4 * c + self.rank], self.w2t, self.w0, w_pre, act="tanh")
         out = self.rt.empty(n, c)
         ops.recurrent_scan(r, k, v, w_pre, g, self.norm_w, self.norm_eps, state[:, h:], ctx.q_start, ctx.positions,
                            ctx.state_slots, out, self.num_heads, self.head_dim, self.rule, bonus=self.bonus)

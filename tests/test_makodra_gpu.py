@@ -81,7 +81,7 @@ def test_lowrank_second_half(ops):
         buf = torch.randn(6, rank + 5)
         w2, b = torch.randn(feats, rank), torch.randn(feats)
         out = torch.empty(6, feats).cuda()
-        ops.lowrank_out(buf.cuda()[:, 5:], w2.cuda(), b.cuda(), out, act="tanh")
+        ops.lowrank_out(buf.cuda()[:, 5:], w2.t().contiguous().cuda(), b.cuda(), out, act="tanh")
         ref = torch.tanh(buf[:, 5:].double()) @ w2.double().T + b.double()
         assert (out.cpu().double() - ref).abs().max() < 1e-5
 
@@ -319,8 +319,10 @@ CONFIGS = {
               "layers": [rec("wkv", 2, 16, 160, rank=8), attn(4, 2, 32, 16, 24, 0.2, True, 0), rec("general_delta", 3, 24, 64, rank=12),
                          attn(2, 2, 48, 16, 7, 0.15, True, 128), attn(6, 1, 16, 40, 0, 0.3, False, 96),
                          attn(4, 2, 32, 16, 50, 0.25, True, 0)]},
-    # a width that the few-row product kernels do not take, single heads, a chunk equal to a page, a tight cap
-    "odd": {"architecture": "Makodra", "vocab": 97, "width": 80, "norm": {"eps": 1e-6}, "logit_softcap": 3.0,
+    # a width that the few-row product kernels do not take, single heads, a chunk equal to a page, a tight cap,
+    # a large eps (with a small one, a head whose first outputs are near zero is normalised to a sign
+    # that rounding decides, and bfloat16 cannot be held to anything there)
+    "odd": {"architecture": "Makodra", "vocab": 97, "width": 80, "norm": {"eps": 1e-2}, "logit_softcap": 3.0,
             "layers": [rec("general_delta", 1, 64, 0), rec("wkv", 5, 16, 72), attn(1, 1, 80, 80, 16, 0.1, True, 40)]},
     # attention only, grouped heads
     "attention": {"architecture": "Makodra", "vocab": 64, "width": 64, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
