@@ -32,7 +32,8 @@ def build_makodra_spec(cfg: MakodraConfig) -> ModelSpec:
                  "mixer_norm": ("norm", PartSpec("rms_norm", dict(width=w, eps=eps, weight_name="norm1"), p))}
         if layer.ff:
             parts["feed_forward"] = ("feed_forward", PartSpec("gated_mlp", dict(
-                hidden_size=w, intermediate_size=layer.ff, names={"gate": "gate", "up": "up", "down": "down"}), p + "mlp."))
+                hidden_size=w, intermediate_size=layer.ff, names={"gate": "gate", "up": "up", "down": "down"},
+                few_rows_fused=True), p + "mlp."))
             parts["feed_forward_norm"] = ("norm", PartSpec("rms_norm", dict(width=w, eps=eps, weight_name="norm2"), p))
         layers.append(LayerSpec(block=PartSpec("output_norm"), parts=parts))
     return ModelSpec(

@@ -9,15 +9,18 @@
 // sigmoid(g_pre) (RULE_DELTA) or silu(g_pre) (RULE_BONUS); the result is written in the type of
 // the product that reads it. Everything here is 32-bit arithmetic on 32-bit inputs.
 //
-// One wave takes one (entry, head, slice of 16 value columns) and walks the entry's tokens in
-// order; waves never wait for each other. Lane (v, part) keeps the D / 4 state values
-// S[part's keys][v] in registers: a column of S never leaves its four neighbouring lanes, whose
-// partial dot products meet in two DPP swaps inside a quad. The per-token vectors of 16 tokens (8 for heads above 64)
-// are staged in LDS at once (the loads of the next batch are in flight while the chain over this
-// batch's tokens runs, and the chain itself reads LDS and registers only). o goes out in 32-bit;
-// a second kernel normalises each head's o and applies the gate (it needs all of a head's
-// columns, which lie in several waves). The sums of a token do not depend on where a step cut the
-// request: the state is the only thing carried, and it is carried exactly.
+// One wave takes one (entry, head, slice of 8 value columns) and walks the entry's tokens in
+// order; waves never wait for each other. Lane (v, part) keeps the D / 8 state values
+// S[part's keys][v] in registers: a column of S never leaves its eight neighbouring lanes, whose
+// partial dot products meet in three DPP swaps. A wave alone on its SIMD issues an instruction
+// every four to five cycles, so the chain over a request's tokens is as long as a token's
+// instructions: eight lanes a column keep that to some hundred. The per-token vectors of 16
+// tokens (8 for heads above 64; one in a step of single tokens) are staged in LDS at once: the
+// loads of the next batch are in flight while the chain over this batch's tokens runs, and the
+// chain itself reads LDS and registers only. o goes out in 32-bit; a second kernel normalises
+// each head's o and applies the gate (it needs all of a head's columns, which lie in several
+// waves). The sums of a token do not depend on where a step cut the request: the state is the
+// only thing carried, and it is carried exactly.
 //
 // State slot layout: [heads][D (value)][D (key)] floats at `state + slot * state_stride`.
 // A request whose first row of the step has position 0 starts from a zero state.
@@ -42,38 +45,40 @@ struct ScanArgs {
   int heads;
 };
 
-// Sum over the four lanes of a quad (every lane gets it), by two DPP quad permutes.
-__device__ __forceinline__ float quad_sum(float x) {
+// Sum over the eight lanes of an octet (every lane gets it): two DPP quad permutes, then the
+// mirror of a half row, which swaps an octet's two quads (whose lanes already agree).
+__device__ __forceinline__ float octet_sum(float x) {
   x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, false));
   x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, false));
+  x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x141, 0xF, 0xF, false));
   return x;
 }
 
-template <int NK, int RULE>
+template <int NK, int RULE, int TB>
 __global__ __launch_bounds__(64) void recurrent_scan_kernel(ScanArgs p) {
-  constexpr int D = NK * 4, TB = D > 64 ? 8 : 16, PER = TB * D / 64;  // PER: what a lane stages per vector and batch
-  __shared__ float sk[TB * D], sw[TB * D], sa[RULE == RULE_DELTA ? TB * D : 1], sr[TB * D];
-  const int lane = threadIdx.x, vloc = lane >> 2, part = lane & 3;
-  const int entry = blockIdx.x, head = blockIdx.y, col = blockIdx.z * 16 + vloc;
-  const bool live = col < D;
-  const int ccol = live ? col : D - 1;
+  constexpr int D = NK * 8, PER = (TB * D + 63) / 64;  // PER: what a lane stages per vector and batch
+  __shared__ float sk[PER * 64], sw[PER * 64], sa[RULE == RULE_DELTA ? PER * 64 : 1], sr[PER * 64];
+  const int lane = threadIdx.x, vloc = lane >> 3, part = lane & 7;
+  const int entry = blockIdx.x, head = blockIdx.y, col = blockIdx.z * 8 + vloc;
   const int row0 = p.q_start[entry], n_rows = p.q_start[entry + 1] - row0;
   if (n_rows <= 0) return;
   const int64_t col0 = (int64_t)head * D;
-  float* st = p.state + (int64_t)p.state_slots[entry] * p.state_stride + ((int64_t)head * D + ccol) * D + part * NK;
+  float* st = p.state + (int64_t)p.state_slots[entry] * p.state_stride + ((int64_t)head * D + col) * D + part * NK;
   float s[NK], bon[NK];
   const bool fresh = p.positions[row0] == 0;
 #pragma unroll
   for (int i = 0; i < NK; ++i) {
-    s[i] = (fresh || !live) ? 0.f : st[i];
+    s[i] = fresh ? 0.f : st[i];
     bon[i] = RULE == RULE_BONUS ? p.bonus[col0 + part * NK + i] : 0.f;
   }
 
-  float pk[PER], pw[PER], pa[PER], pr[PER], pv[TB];
+  constexpr int PV = (TB * 8 + 63) / 64;
+  __shared__ float sv[PV * 64], skn[TB];
+  float pk[PER], pw[PER], pa[PER], pr[PER], pv[PV];
   auto fetch = [&](int t0) {
 #pragma unroll
     for (int m = 0; m < PER; ++m) {
-      const int e = lane + 64 * m, t = e / D, c = e - t * D;
+      const int e = min(lane + 64 * m, TB * D - 1), t = e / D, c = e - t * D;
       const int64_t row = row0 + min(t0 + t, n_rows - 1);
       pk[m] = p.k[row * p.k_stride + col0 + c];
       pr[m] = p.r[row * p.r_stride + col0 + c];
@@ -81,11 +86,46 @@ __global__ __launch_bounds__(64) void recurrent_scan_kernel(ScanArgs p) {
       if (RULE == RULE_DELTA) pa[m] = p.a_pre[row * p.a_stride + col0 + c] + p.a_bias[col0 + c];
     }
 #pragma unroll
-    for (int t = 0; t < TB; ++t) pv[t] = p.v[(int64_t)(row0 + min(t0 + t, n_rows - 1)) * p.v_stride + col0 + ccol];
+    for (int m = 0; m < PV; ++m) {
+      const int e = min(lane + 64 * m, TB * 8 - 1);
+      pv[m] = p.v[(int64_t)(row0 + min(t0 + e / 8, n_rows - 1)) * p.v_stride + col0 + blockIdx.z * 8 + e % 8];
+    }
+  };
+  // One token of the chain, from LDS and registers only. Nothing but s hangs on the token before:
+  // the reads of the next tokens can be issued while this one's sums are made.
+  auto step = [&](int t, int64_t row) {
+    const float* kt = sk + t * D + part * NK;
+    const float* wt = sw + t * D + part * NK;
+    const float* rt = sr + t * D + part * NK;
+    const float v = sv[t * 8 + vloc];
+    float o0 = 0.f, o1 = 0.f;
+    if (RULE == RULE_DELTA) {
+      const float* at = sa + t * D + part * NK;
+      const float kn = skn[t];
+      float ks0 = 0.f, ks1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < NK; ++i) {
+        if (i & 1) ks1 = fmaf(kt[i], s[i], ks1); else ks0 = fmaf(kt[i], s[i], ks0);
+      }
+      const float us = octet_sum(ks0 + ks1) * kn;       // u^T S for this column, u = k * kn
+#pragma unroll
+      for (int i = 0; i < NK; ++i) {
+        s[i] = wt[i] * s[i] - (at[i] * (kt[i] * kn)) * us + kt[i] * v;
+        if (i & 1) o1 = fmaf(s[i], rt[i], o1); else o0 = fmaf(s[i], rt[i], o0);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NK; ++i) {
+        const float kv = kt[i] * v;
+        if (i & 1) o1 = fmaf(s[i] + bon[i] * kv, rt[i], o1); else o0 = fmaf(s[i] + bon[i] * kv, rt[i], o0);
+        s[i] = wt[i] * s[i] + kv;
+      }
+    }
+    const float o = octet_sum(o0 + o1);
+    if (part == 0) p.o_raw[row * p.o_stride + col0 + col] = o;
   };
   fetch(0);
   for (int t0 = 0; t0 < n_rows; t0 += TB) {
-    float vv[TB];
 #pragma unroll
     for (int m = 0; m < PER; ++m) {
       const int e = lane + 64 * m;
@@ -99,56 +139,31 @@ __global__ __launch_bounds__(64) void recurrent_scan_kernel(ScanArgs p) {
       }
     }
 #pragma unroll
-    for (int t = 0; t < TB; ++t) vv[t] = live ? pv[t] : 0.f;
-    if (t0 + TB < n_rows) fetch(t0 + TB);  // on their way while the chain below runs
-    __syncthreads();                       // (one wave: orders its LDS writes before its reads)
-    const int nb = min(TB, n_rows - t0);
-#pragma unroll
-    for (int t = 0; t < TB; ++t) {
-      if (t < nb) {
-        const float* kt = sk + t * D + part * NK;
-        const float* wt = sw + t * D + part * NK;
-        const float* rt = sr + t * D + part * NK;
-        float o0 = 0.f, o1 = 0.f;
-        if (RULE == RULE_DELTA) {
-          const float* at = sa + t * D + part * NK;
-          float ks0 = 0.f, ks1 = 0.f, kk = 0.f;
-#pragma unroll
-          for (int i = 0; i < NK; i += 2) {
-            ks0 = fmaf(kt[i], s[i], ks0);
-            ks1 = fmaf(kt[i + 1], s[i + 1], ks1);
-            kk = fmaf(kt[i], kt[i], kk);
-            kk = fmaf(kt[i + 1], kt[i + 1], kk);
-          }
-          const float kn = 1.f / sqrtf(quad_sum(kk) + 1e-6f);
-          const float us = quad_sum(ks0 + ks1) * kn;       // u^T S for this column, u = k * kn
-#pragma unroll
-          for (int i = 0; i < NK; i += 2) {
-            s[i] = wt[i] * s[i] - (at[i] * (kt[i] * kn)) * us + kt[i] * vv[t];
-            s[i + 1] = wt[i + 1] * s[i + 1] - (at[i + 1] * (kt[i + 1] * kn)) * us + kt[i + 1] * vv[t];
-            o0 = fmaf(s[i], rt[i], o0);
-            o1 = fmaf(s[i + 1], rt[i + 1], o1);
-          }
-        } else {
-#pragma unroll
-          for (int i = 0; i < NK; i += 2) {
-            const float kv0 = kt[i] * vv[t], kv1 = kt[i + 1] * vv[t];
-            o0 = fmaf(s[i] + bon[i] * kv0, rt[i], o0);
-            o1 = fmaf(s[i + 1] + bon[i + 1] * kv1, rt[i + 1], o1);
-            s[i] = wt[i] * s[i] + kv0;
-            s[i + 1] = wt[i + 1] * s[i + 1] + kv1;
-          }
-        }
-        const float o = quad_sum(o0 + o1);
-        if (part == 0 && live) p.o_raw[(int64_t)(row0 + t0 + t) * p.o_stride + col0 + col] = o;
+    for (int m = 0; m < PV; ++m) sv[lane + 64 * m] = pv[m];
+    if (TB > 1 && t0 + TB < n_rows) fetch(t0 + TB);  // on their way while the chain below runs
+    __syncthreads();                                 // (one wave: orders its LDS writes before its reads)
+    if (RULE == RULE_DELTA) {
+      // each token's 1 / sqrt(sum k^2 + 1e-6): four lanes a token add up a quarter of its keys each
+      for (int t = lane >> 2; t < TB; t += 16) {
+        float kk = 0.f;
+        for (int c = (lane & 3) * (D / 4); c < ((lane & 3) + 1) * (D / 4); ++c) kk = fmaf(sk[t * D + c], sk[t * D + c], kk);
+        kk += __shfl_xor(kk, 1, DLI_WAVE);
+        kk += __shfl_xor(kk, 2, DLI_WAVE);
+        if ((lane & 3) == 0) skn[t] = 1.f / sqrtf(kk + 1e-6f);
       }
+      __syncthreads();
+    }
+    const int nb = min(TB, n_rows - t0);
+    if (nb == TB) {
+#pragma unroll
+      for (int t = 0; t < TB; ++t) step(t, row0 + t0 + t);
+    } else {
+      for (int t = 0; t < nb; ++t) step(t, row0 + t0 + t);
     }
     __syncthreads();  // the chain has read this batch before the next one is written
   }
-  if (live) {
 #pragma unroll
-    for (int i = 0; i < NK; ++i) st[i] = s[i];
-  }
+  for (int i = 0; i < NK; ++i) st[i] = s[i];
 }
 
 // out = o / sqrt(mean_head(o^2) + eps) * norm_w * gate(g_pre), head by head: one workgroup a row,
@@ -175,12 +190,17 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
 
 template <int RULE>
 static int launch_scan(const ScanArgs& p, int entries, int rows, int dim, int out_is_bf16, hipStream_t stream) {
-  const dim3 grid(entries, p.heads, (dim + 15) / 16);
-#define SCAN_CASE(NK) \
-  case NK: recurrent_scan_kernel<NK, RULE><<<grid, 64, 0, stream>>>(p); break;
-  switch (dim / 4) {
-    SCAN_CASE(4) SCAN_CASE(6) SCAN_CASE(8) SCAN_CASE(10) SCAN_CASE(12) SCAN_CASE(14) SCAN_CASE(16)
-    SCAN_CASE(20) SCAN_CASE(24) SCAN_CASE(28) SCAN_CASE(32)
+  const dim3 grid(entries, p.heads, dim / 8);
+  // a step of single tokens stages one token a wave; any other stages 16 (8 for heads above 64)
+  const bool single = rows == entries;
+#define SCAN_CASE(NK, TBM)                                                                           \
+  case NK:                                                                                           \
+    if (single) recurrent_scan_kernel<NK, RULE, 1><<<grid, 64, 0, stream>>>(p);                      \
+    else recurrent_scan_kernel<NK, RULE, TBM><<<grid, 64, 0, stream>>>(p);                           \
+    break;
+  switch (dim / 8) {
+    SCAN_CASE(2, 16) SCAN_CASE(3, 16) SCAN_CASE(4, 16) SCAN_CASE(5, 16) SCAN_CASE(6, 16) SCAN_CASE(7, 16)
+    SCAN_CASE(8, 16) SCAN_CASE(10, 8) SCAN_CASE(12, 8) SCAN_CASE(14, 8) SCAN_CASE(16, 8)
     default: return DLI_ERR_ARGUMENT;
   }
 #undef SCAN_CASE
@@ -209,7 +229,7 @@ extern "C" int dli_recurrent_scan(const float* r, int64_t r_stride, const float*
                                   int64_t out_stride, int entries, int rows, int heads, int dim, int rule,
                                   int out_is_bf16, hipStream_t stream) {
   if (entries <= 0 || rows <= 0) return DLI_OK;
-  if (!dli_recurrent_scan_supports(dim) || heads <= 0 || heads > 65535 || (rule != RULE_DELTA && rule != RULE_BONUS) ||
+  if (rows < entries || !dli_recurrent_scan_supports(dim) || heads <= 0 || heads > 65535 || (rule != RULE_DELTA && rule != RULE_BONUS) ||
       state_stride < (int64_t)heads * dim * dim || (rule == RULE_DELTA && (a_pre == nullptr || a_bias == nullptr)) ||
       (rule == RULE_BONUS && bonus == nullptr))
     return DLI_ERR_ARGUMENT;

@@ -5,7 +5,8 @@
 //
 //   embed_sinusoid     x = table[id] + pe(position), pe[2i] = sin(p f_i), pe[2i+1] = cos(p f_i)
 //   cast_from_f32      the stream rounded to T, as the operand of a product
-//   norm_into_stream   x += w * y / sqrt(mean(y^2) + eps)   (a norm on a sublayer's output)
+//   norm_into_stream   x += w * y / sqrt(mean(y^2) + eps)   (a norm on a sublayer's output); like the embedding
+//                      it can leave the new stream once more in bf16, for the product that reads it next
 //   rms_norm_from_f32  out(T) = w * x / sqrt(mean(x^2) + eps)
 //   softcap            y = cap * tanh(y / cap)
 //   token_shift        S mixes of each row with the row before it, x + (prev - x) * mu_s; the row
@@ -18,13 +19,15 @@
 template <typename T>
 __global__ void embed_sinusoid_kernel(const T* __restrict__ table, const int* __restrict__ ids,
                                       const int* __restrict__ positions, const float* __restrict__ inv_freq,
-                                      float* __restrict__ out, int width) {
+                                      float* __restrict__ out, bf16_t* __restrict__ rounded, int width) {
   const int64_t row = blockIdx.x;
   const T* src = table + (int64_t)ids[row] * width;
   const float p = (float)positions[row];
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     const float angle = p * inv_freq[i >> 1];
-    out[row * width + i] = to_f32(src[i]) + ((i & 1) ? cosf(angle) : sinf(angle));
+    const float sum = to_f32(src[i]) + ((i & 1) ? cosf(angle) : sinf(angle));
+    out[row * width + i] = sum;
+    if (rounded != nullptr) rounded[row * width + i] = (bf16_t)sum;
   }
 }
 
@@ -34,9 +37,10 @@ __global__ void cast_from_f32_kernel(const float* __restrict__ x, T* __restrict_
   if (i < n) out[i] = from_f32<T>(x[i]);
 }
 
-template <typename T>
+// `rounded` (may be nullptr): the new stream once more in type R, for the product that reads it next.
+template <typename T, typename R>
 __global__ void norm_into_stream_kernel(const T* __restrict__ y, int64_t y_stride, const float* __restrict__ weight,
-                                        float* __restrict__ x, int width, float eps) {
+                                        float* __restrict__ x, R* __restrict__ rounded, int width, float eps) {
   __shared__ float scratch[16];
   const int64_t row = blockIdx.x;
   const T* yr = y + row * y_stride;
@@ -47,7 +51,11 @@ __global__ void norm_into_stream_kernel(const T* __restrict__ y, int64_t y_strid
   }
   const float r = 1.f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
   float* xr = x + row * width;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) xr[i] += weight[i] * (to_f32(yr[i]) * r);
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float sum = xr[i] + weight[i] * (to_f32(yr[i]) * r);
+    xr[i] = sum;
+    if (rounded != nullptr) rounded[row * width + i] = from_f32<R>(sum);
+  }
 }
 
 template <typename T>
@@ -118,11 +126,20 @@ __global__ void lowrank_out_kernel(const float* __restrict__ t, int64_t t_stride
     ts[j] = act == 1 ? tanhf(v) : v;
   }
   __syncthreads();
-  for (int c = threadIdx.x; c < features; c += blockDim.x) {
-    float s = 0.f;
-    for (int j = 0; j < rank; ++j) s = fmaf(ts[j], w2t[(int64_t)j * features + c], s);
-    out[row * features + c] = s + (bias != nullptr ? bias[c] : 0.f);
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;   // a feature a thread
+  if (c >= features) return;
+  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;          // four sums: the weights' loads do not wait for each other
+  int j = 0;
+  for (; j + 4 <= rank; j += 4) {
+    const float a = w2t[(int64_t)j * features + c], b = w2t[(int64_t)(j + 1) * features + c];
+    const float d = w2t[(int64_t)(j + 2) * features + c], e = w2t[(int64_t)(j + 3) * features + c];
+    s0 = fmaf(ts[j], a, s0);
+    s1 = fmaf(ts[j + 1], b, s1);
+    s2 = fmaf(ts[j + 2], d, s2);
+    s3 = fmaf(ts[j + 3], e, s3);
   }
+  for (; j < rank; ++j) s0 = fmaf(ts[j], w2t[(int64_t)j * features + c], s0);
+  out[row * features + c] = ((s0 + s1) + (s2 + s3)) + (bias != nullptr ? bias[c] : 0.f);
 }
 
 // proj [tokens][stride] float32 holds q (q_heads x dim), k (kv_heads x dim) and v (kv_heads x vdim)
@@ -171,14 +188,16 @@ __global__ void qk_unit_cache_kernel(const float* __restrict__ proj, int64_t str
 extern "C" {
 
 int dli_embed_sinusoid(const void* table, const int* ids, const int* positions, const float* inv_freq, float* out,
-                       int rows, int width, int is_bf16, hipStream_t stream) {
+                       void* rounded_bf16, int rows, int width, int is_bf16, hipStream_t stream) {
   if (rows <= 0) return DLI_OK;
   if (width <= 0) return DLI_ERR_ARGUMENT;
   const int threads = width >= 1024 ? 256 : 128;
   if (is_bf16)
-    embed_sinusoid_kernel<bf16_t><<<rows, threads, 0, stream>>>((const bf16_t*)table, ids, positions, inv_freq, out, width);
+    embed_sinusoid_kernel<bf16_t><<<rows, threads, 0, stream>>>((const bf16_t*)table, ids, positions, inv_freq, out,
+                                                                (bf16_t*)rounded_bf16, width);
   else
-    embed_sinusoid_kernel<float><<<rows, threads, 0, stream>>>((const float*)table, ids, positions, inv_freq, out, width);
+    embed_sinusoid_kernel<float><<<rows, threads, 0, stream>>>((const float*)table, ids, positions, inv_freq, out,
+                                                               (bf16_t*)rounded_bf16, width);
   return dli_launch_status();
 }
 
@@ -191,15 +210,17 @@ int dli_cast_from_f32(const float* x, void* out, int64_t n, int is_bf16, hipStre
   return dli_launch_status();
 }
 
-int dli_norm_into_stream(const void* y, int64_t y_stride, const float* weight, float* x, int rows, int width, float eps,
-                         int y_is_bf16, hipStream_t stream) {
+int dli_norm_into_stream(const void* y, int64_t y_stride, const float* weight, float* x, void* rounded_bf16, int rows,
+                         int width, float eps, int y_is_bf16, hipStream_t stream) {
   if (rows <= 0) return DLI_OK;
   if (width <= 0 || y_stride < width) return DLI_ERR_ARGUMENT;
   const int threads = width >= 2048 ? 512 : 256;
   if (y_is_bf16)
-    norm_into_stream_kernel<bf16_t><<<rows, threads, 0, stream>>>((const bf16_t*)y, y_stride, weight, x, width, eps);
+    norm_into_stream_kernel<bf16_t, bf16_t><<<rows, threads, 0, stream>>>((const bf16_t*)y, y_stride, weight, x,
+                                                                          (bf16_t*)rounded_bf16, width, eps);
   else
-    norm_into_stream_kernel<float><<<rows, threads, 0, stream>>>((const float*)y, y_stride, weight, x, width, eps);
+    norm_into_stream_kernel<float, bf16_t><<<rows, threads, 0, stream>>>((const float*)y, y_stride, weight, x,
+                                                                         (bf16_t*)rounded_bf16, width, eps);
   return dli_launch_status();
 }
 
@@ -242,7 +263,8 @@ int dli_lowrank_out(const float* t, int64_t t_stride, const float* w2t, const fl
                     int features, int rank, int act, hipStream_t stream) {
   if (rows <= 0) return DLI_OK;
   if (features <= 0 || rank <= 0 || rank > 8192 || t_stride < rank || act < 0 || act > 1) return DLI_ERR_ARGUMENT;
-  lowrank_out_kernel<<<rows, 256, rank * sizeof(float), stream>>>(t, t_stride, w2t, bias, out, features, rank, act);
+  lowrank_out_kernel<<<dim3(rows, (features + 255) / 256), 256, rank * sizeof(float), stream>>>(t, t_stride, w2t, bias, out,
+                                                                                                features, rank, act);
   return dli_launch_status();
 }
 

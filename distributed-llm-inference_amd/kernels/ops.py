@@ -100,9 +100,9 @@ _SIGNATURES = {
     "dli_attention_scored": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr,
                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_ptr,
                              _c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr],
-    "dli_embed_sinusoid": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_embed_sinusoid": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "dli_cast_from_f32": [_c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr],
-    "dli_norm_into_stream": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+    "dli_norm_into_stream": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "dli_rms_norm_from_f32": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "dli_softcap": [_c_ptr, _c_i64, _c_float, _c_ptr],
     "dli_token_shift": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
@@ -1334,10 +1334,18 @@ def _f32_rows(t: torch.Tensor, name: str) -> None:
     _rows(t, name, torch.float32)
 
 
+def _rounded_copy(rounded: Optional[torch.Tensor], like: torch.Tensor) -> None:
+    if rounded is not None:
+        _dense(rounded, "rounded", torch.bfloat16, 2)
+        _require(rounded.shape == like.shape, "the rounded copy differs from the stream in shape")
+
+
 def embed_sinusoid(table: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor,
-                   out: torch.Tensor) -> None:
+                   out: torch.Tensor, rounded: Optional[torch.Tensor] = None) -> None:
     """``out[t] = table[ids[t]] + pe(positions[t])`` in float32, ``pe[2i] = sin(p f_i)``,
-    ``pe[2i+1] = cos(p f_i)`` with ``f = inv_freq [ceil(width/2)]``."""
+    ``pe[2i+1] = cos(p f_i)`` with ``f = inv_freq [ceil(width/2)]``. ``rounded``: the same rows once
+    more in bfloat16."""
+    _rounded_copy(rounded, out)
     _dense(table, "table", ndim=2)
     _dense(ids, "ids", torch.int32, 1)
     _dense(positions, "positions", torch.int32, 1)
@@ -1346,7 +1354,7 @@ def embed_sinusoid(table: torch.Tensor, ids: torch.Tensor, positions: torch.Tens
     n, width = ids.shape[0], table.shape[1]
     _require(positions.shape[0] == n and out.shape == (n, width), "ids, positions and out disagree on the rows")
     _require(inv_freq.shape[0] * 2 >= width, "inv_freq must hold a frequency for every pair of columns")
-    _check(library().dli_embed_sinusoid(_ptr(table), _ptr(ids), _ptr(positions), _ptr(inv_freq), _ptr(out), n, width,
+    _check(library().dli_embed_sinusoid(_ptr(table), _ptr(ids), _ptr(positions), _ptr(inv_freq), _ptr(out), _ptr(rounded), n, width,
                                         _is_bf16(table.dtype), _stream()), "embed_sinusoid")
 
 
@@ -1358,14 +1366,17 @@ def cast_from_f32(x: torch.Tensor, out: torch.Tensor) -> None:
     _check(library().dli_cast_from_f32(_ptr(x), _ptr(out), x.numel(), _is_bf16(out.dtype), _stream()), "cast_from_f32")
 
 
-def norm_into_stream(y: torch.Tensor, weight: torch.Tensor, eps: float, x: torch.Tensor) -> None:
+def norm_into_stream(y: torch.Tensor, weight: torch.Tensor, eps: float, x: torch.Tensor,
+                     rounded: Optional[torch.Tensor] = None) -> None:
     """``x += weight * y / sqrt(mean(y^2) + eps)`` row by row: ``x`` float32 ``[n, width]``, ``y`` float32
-    or bfloat16 with contiguous rows, statistics and sum in 32-bit."""
+    or bfloat16 with contiguous rows, statistics and sum in 32-bit. ``rounded``: the new ``x`` once more
+    in bfloat16 (what the next product reads)."""
+    _rounded_copy(rounded, x)
     _rows(y, "y", y.dtype)
     _dense(x, "x", torch.float32, 2)
     _dense(weight, "weight", torch.float32, 1)
     _require(y.shape == x.shape and weight.shape[0] == x.shape[1], "y, x and weight disagree on the sizes")
-    _check(library().dli_norm_into_stream(_ptr(y), y.stride(0), _ptr(weight), _ptr(x), x.shape[0], x.shape[1],
+    _check(library().dli_norm_into_stream(_ptr(y), y.stride(0), _ptr(weight), _ptr(x), _ptr(rounded), x.shape[0], x.shape[1],
                                           float(eps), _is_bf16(y.dtype), _stream()), "norm_into_stream")
 
 

@@ -90,9 +90,11 @@ class OutputNormBlock(Block):
             raise RuntimeError("the output_norm block keeps a float32 residual stream")
         if delta is not None:
             from ..kernels import ops
+            from .linear import RoundedStream
             ops.add(x, delta, x)
-        parts["mixer_norm"].add_normed(x, parts["mixer"].forward(x, ctx, cache))
+            RoundedStream.offer(ctx, x, None)
+        parts["mixer_norm"].add_normed(x, parts["mixer"].forward(x, ctx, cache), ctx)
         if "feed_forward" in parts:
-            y = parts["feed_forward"].forward(as_operand(self.rt, x), ctx)
-            parts["feed_forward_norm"].add_normed(x, y)
+            y = parts["feed_forward"].forward(as_operand(self.rt, x, ctx), ctx)
+            parts["feed_forward_norm"].add_normed(x, y, ctx)
         return x, None

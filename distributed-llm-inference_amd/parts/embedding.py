@@ -83,6 +83,10 @@ class SinusoidalTokenEmbedding(TokenEmbedding):
     def forward_step(self, ctx: Any) -> torch.Tensor:
         if self._inv_freq is None:
             self.finalize()
+        from .linear import RoundedStream
+
         out = torch.empty(ctx.token_ids.shape[0], self.hidden_size, device=self.rt.device, dtype=torch.float32)
-        ops.embed_sinusoid(self.table(), ctx.token_ids, ctx.positions, self._inv_freq, out)
+        rounded = self.rt.empty(*out.shape) if self.rt.is_bf16 and hasattr(ctx, "_memo") else None
+        ops.embed_sinusoid(self.table(), ctx.token_ids, ctx.positions, self._inv_freq, out, rounded=rounded)
+        RoundedStream.offer(ctx, out, rounded)
         return out

@@ -20,8 +20,12 @@ class GatedMLP(FeedForward):
     NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
 
     def __init__(self, runtime: Runtime, *, hidden_size: int, intermediate_size: int,
-                 activation: str = "silu", bias: bool = False, names: Optional[Mapping[str, str]] = None) -> None:
+                 activation: str = "silu", bias: bool = False, names: Optional[Mapping[str, str]] = None,
+                 few_rows_fused: bool = False) -> None:
         super().__init__(runtime)
+        # forward() itself takes the few-row kernels (SwiGLU inside the first product) for up to 16
+        # rows: for blocks that have no fused decode path of their own
+        self.few_rows_fused = bool(few_rows_fused)
         # checkpoint names of the three matrices below the part's prefix, where they are not the usual ones
         self.names = {**self.NAMES, **dict(names or {})}
         if bias and names:
@@ -68,6 +72,19 @@ class GatedMLP(FeedForward):
                 "hidden": h, "intermediate": i}
 
     def forward(self, x: torch.Tensor, ctx: Any) -> torch.Tensor:
+        n = x.shape[0]
+        if (self.few_rows_fused and self.rt.is_bf16 and 0 < n <= self.FEW_ROWS and x.dtype == torch.bfloat16 and x.stride(0) % 8 == 0
+                and x.data_ptr() % 16 == 0 and ops.skinny_gemm_supports(n, self.hidden_size, x.dtype)
+                and ops.skinny_gemm_supports(n, self.intermediate_size, x.dtype)):
+            # a few rows outside the fused decode path (a block that keeps its stream in 32-bit, say):
+            # the few-row products, SwiGLU inside the first
+            act = self.rt.empty(n, self.intermediate_size)
+            ops.skinny_gemm(x, self.w_gate_up, w_tiled=self.w_gate_up_tiled, epilogue=ops.SKINNY_SWIGLU, out=act,
+                            bias=self.b_gate_up)
+            out = self.rt.empty(n, self.hidden_size)
+            ops.skinny_gemm(act, self.w_down, w_tiled=self.w_down_tiled, epilogue=ops.SKINNY_STORE, out=out,
+                            bias=self.b_down)
+            return out
         gate_up = linear(self.rt, x, self.w_gate_up, self.b_gate_up)
         act = self.rt.empty(x.shape[0], self.intermediate_size)
         ops.silu_mul(gate_up, act)

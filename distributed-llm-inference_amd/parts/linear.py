@@ -78,13 +78,39 @@ def finish_residual(rt: Runtime, stream: DecodeStream, partial: torch.Tensor, bi
         stream.wrote(ops.mid_finish_residual(partial, stream.x, bias))
 
 
-def as_operand(rt: Runtime, x: torch.Tensor) -> torch.Tensor:
+class RoundedStream:
+    """The rounded copy of a 32-bit residual stream that the kernel which last wrote the stream
+    left beside it (the embedding, a norm that adds into the stream): whoever reads the stream as
+    a product's operand next takes it instead of rounding the stream once more. It is kept on the
+    step's context under the stream's address and dropped by whoever changes the stream."""
+
+    KEY = "rounded stream"
+
+    @staticmethod
+    def offer(ctx, x: torch.Tensor, rounded: Optional[torch.Tensor]) -> None:
+        if ctx is not None and hasattr(ctx, "_memo"):
+            if rounded is None:
+                ctx._memo.pop(RoundedStream.KEY, None)
+            else:
+                ctx._memo[RoundedStream.KEY] = (x.data_ptr(), tuple(x.shape), rounded)
+
+    @staticmethod
+    def take(ctx, x: torch.Tensor) -> Optional[torch.Tensor]:
+        hit = getattr(ctx, "_memo", {}).get(RoundedStream.KEY) if ctx is not None else None
+        return hit[2] if hit is not None and hit[:2] == (x.data_ptr(), tuple(x.shape)) else None
+
+
+def as_operand(rt: Runtime, x: torch.Tensor, ctx=None) -> torch.Tensor:
     """``x`` in the type that the runtime's products read: a 32-bit residual stream is rounded to
-    bfloat16 when serving and used as it is on the 32-bit path."""
+    bfloat16 when serving (or its rounded copy is taken from ``ctx`` where its last writer left
+    one) and used as it is on the 32-bit path."""
     if x.dtype == rt.dtype:
         return x
     if x.dtype != torch.float32:
         raise ops.KernelArgumentError(f"an operand of type {x.dtype} in a runtime of {rt.dtype}")
+    ready = RoundedStream.take(ctx, x)
+    if ready is not None:
+        return ready
     out = rt.empty(*x.shape)
     ops.cast_from_f32(x, out)
     return out

@@ -41,10 +41,16 @@ class RMSNorm(Norm):
             return None
         return {"kind": "rms_norm", "w": w, "eps": self.eps, "width": self.width}
 
-    def add_normed(self, x: torch.Tensor, y: torch.Tensor) -> None:
+    def add_normed(self, x: torch.Tensor, y: torch.Tensor, ctx=None) -> None:
         """``x += norm(y)``: the norm on a sublayer's output, added into a 32-bit residual stream
-        ``x`` in one kernel (statistics, product and sum in 32-bit; ``y`` float32 or bfloat16)."""
-        ops.norm_into_stream(y, self.weight, self.eps, x)
+        ``x`` in one kernel (statistics, product and sum in 32-bit; ``y`` float32 or bfloat16). In a
+        bfloat16 runtime the kernel leaves the new stream once more in bfloat16 on ``ctx``, for the
+        product that reads it next."""
+        from .linear import RoundedStream
+
+        rounded = self.rt.empty(*x.shape) if self.rt.is_bf16 and ctx is not None else None
+        ops.norm_into_stream(y, self.weight, self.eps, x, rounded=rounded)
+        RoundedStream.offer(ctx, x, rounded)
 
     def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None) -> torch.Tensor:
         if x.dtype == torch.float32 and self.rt.is_bf16:

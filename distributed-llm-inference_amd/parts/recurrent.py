@@ -96,7 +96,7 @@ class GeneralDelta(_MatrixStateMixer):
     def forward(self, x: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:
         state = self._check(cache)
         n, c = x.shape[0], self.width
-        proj = linear_f32(self.rt, as_operand(self.rt, x), self.w_in)
+        proj = linear_f32(self.rt, as_operand(self.rt, x, ctx), self.w_in)
         r, k, v, g, a = (proj[:, i * c:(i + 1) * c] for i in range(5))
         w_pre = torch.empty(n, c, device=self.rt.device, dtype=torch.float32)
         ops.lowrank_out(proj[:, 5 * c:5 * c + self.rank], self.w2t, self.w0, w_pre, act="tanh")

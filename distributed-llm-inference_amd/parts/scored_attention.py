@@ -119,7 +119,7 @@ class ScoredAttention(Mixer):
             raise RuntimeError("scored_attention needs a paged cache of its own")
         grp = ctx.groups[cache.group]
         n = x.shape[0]
-        proj = linear_f32(self.rt, as_operand(self.rt, x), self.w_in)
+        proj = linear_f32(self.rt, as_operand(self.rt, x, ctx), self.w_in)
         q = self.rt.empty(n, self._q)
         first_in = first_out = None
         if self.value_mix == "source":
