@@ -284,10 +284,15 @@ def design_compare(args):
             engine, cfg = make_engine(raw, args.dtype, 64, args.context, args.block_size, budget=8192,
                                       decode_steps=args.decode_steps)
             got = {}
+            phases = args.design_phases.split(",")
             for n in (2048, 8192):
+                if f"prefill{n}" not in phases:
+                    continue
                 t = prefill_run(engine, cfg, n, repeats=2)
                 got[f"prefill{n}_tok_s"], got[f"prefill{n}_ms"] = round(n / t, 1), round(t * 1e3, 3)
             for b in (1, 8, 64):
+                if f"decode_b{b}" not in phases:
+                    continue
                 tok_s, ms, _ = decode_run(engine, cfg, b, args.context, min(args.steps, 32), min(args.warmup, 4),
                                           args.decode_steps)
                 got[f"decode_b{b}_tok_s"], got[f"decode_b{b}_ms"] = round(tok_s, 1), round(ms, 4)
@@ -388,6 +393,8 @@ def main() -> int:
                     help="instead of the default run: prefill (2,048 and 8,192 tokens) and decode (batch 1, 8, 64 at "
                          "--context) of this design beside the Llama decoder at equal sizes, random weights")
     ap.add_argument("--design-sizes", default="1024,2048", help="widths of --design, of " + ", ".join(DESIGN_SIZES))
+    ap.add_argument("--design-phases", default="prefill2048,prefill8192,decode_b1,decode_b8,decode_b64",
+                    help="with --design: which of these measurements to make")
     ap.add_argument("--design-only", default=None, choices=["makodra", "llama"],
                     help="with --design: measure this one of the pair alone (for profiling)")
     args = ap.parse_args()

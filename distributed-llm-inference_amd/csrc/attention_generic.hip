@@ -214,19 +214,19 @@ static int launch_generic(const void* q, int64_t q_stride, const void* k_pages, 
 
 // ---------------------------------------------------------------------------------------------
 // Steps of single tokens: one workgroup takes one (entry, kv head, group of up to GQ query heads
-// that share it) and its four waves take the blocks of 64 visible keys in turn. In a block, lane j
+// that share it) and its waves (eight, or four) take the blocks of 64 visible keys in turn. In a block, lane j
 // owns key j: it reads the key's row (16 bytes at a time) and makes its GQ scores against the
 // queries in LDS, the changes to the scores are applied, and each head's reference point moves to
 // the block's maximum (one wave reduction a head); the weights then go through LDS and the lanes
 // change roles: lane c owns value column c (+ 64, ...) and adds up the block's 64 keys, whose
-// values lie side by side in a page's row. The four waves' states are merged through LDS at the
+// values lie side by side in a page's row. The waves' states are merged through LDS at the
 // end. The same arithmetic as the tile kernel, in another order: 32-bit throughout.
 template <typename T> struct Pack16;   // what 16 bytes hold
 template <> struct Pack16<bf16_t> { static constexpr int N = 8; typedef __bf16 type __attribute__((ext_vector_type(8))); };
 template <> struct Pack16<float> { static constexpr int N = 4; typedef float type __attribute__((ext_vector_type(4))); };
 
 template <typename T, int GQ, int VC>
-__global__ __launch_bounds__(256) void attention_scored_decode_kernel(
+__global__ __launch_bounds__(512) void attention_scored_decode_kernel(
     const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     T* __restrict__ out, int64_t out_stride, const int* __restrict__ kv_len, const int* __restrict__ block_tables,
     int table_stride, int q_heads, int kv_heads, int head_dim, int page_size, float scale, int window,
@@ -235,11 +235,11 @@ __global__ __launch_bounds__(256) void attention_scored_decode_kernel(
   typedef typename Pack16<T>::type P16;
   extern __shared__ float lds[];
   const int value_dim = sc.value_dim;
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64, waves = blockDim.x / 64, threads = blockDim.x;
   float* qs = lds;                               // [GQ][head_dim]
-  float* ps = qs + GQ * head_dim;                // [4][GQ][64]
-  float* ms = ps + 4 * GQ * 64;                  // [4][GQ] reference points, then [4][GQ] sums
-  float* accs = ms + 8 * GQ;                     // [4][GQ][VC * 64]
-  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  float* ps = qs + GQ * head_dim;                // [waves][GQ][64]
+  float* ms = ps + waves * GQ * 64;              // [waves][GQ] reference points, then [waves][GQ] sums
+  float* accs = ms + 2 * waves * GQ;             // [waves][GQ][VC * 64]
   const int entry = blockIdx.x, kvh = blockIdx.y;
   const int group = q_heads / kv_heads;
   const int h0 = kvh * group + blockIdx.z * GQ;                  // first query head of this workgroup
@@ -248,7 +248,7 @@ __global__ __launch_bounds__(256) void attention_scored_decode_kernel(
   const int pos = n_keys - 1;
   const int* table = block_tables + (int64_t)entry * table_stride;
 
-  for (int idx = tid; idx < GQ * head_dim; idx += 256) {
+  for (int idx = tid; idx < GQ * head_dim; idx += threads) {
     const int h = idx / head_dim, c = idx - h * head_dim;
     qs[idx] = h < nh ? to_f32(q[(int64_t)entry * q_stride + (int64_t)(h0 + h) * head_dim + c]) * scale : 0.f;
   }
@@ -268,14 +268,17 @@ __global__ __launch_bounds__(256) void attention_scored_decode_kernel(
   __syncthreads();
 
   const bool k_packs = head_dim % PN == 0, v_packs = page_size % PN == 0;
-  for (int j0 = j_begin / 64 * 64 + wave * 64; j0 <= pos; j0 += 256) {
+  for (int j0 = j_begin / 64 * 64 + wave * 64; j0 <= pos; j0 += 64 * waves) {
     const int j = j0 + lane;
     const bool seen = j >= j_begin && j <= pos;
+    // the page of this lane's key, for its own row of K and, handed round, for the rows of V (a key
+    // past the request's last page reads the table's last entry: its weight is zero)
+    const int my_page = table[min(j / page_size, table_stride - 1)];
     float s[GQ];
 #pragma unroll
     for (int h = 0; h < GQ; ++h) s[h] = 0.f;
     if (seen) {
-      const int64_t page = table[j / page_size];
+      const int64_t page = my_page;
       const T* kr = k_pages + ((page * kv_heads + kvh) * page_size + j % page_size) * head_dim;
       if (k_packs) {
         for (int d = 0; d < head_dim; d += PN) {
@@ -316,6 +319,32 @@ __global__ __launch_bounds__(256) void attention_scored_decode_kernel(
     // lanes are value columns now
     const int last = min(63, pos - j0);
     const int first = max(0, j_begin - j0);
+    if (v_packs) {
+      // every pack of the block's 64 keys is asked for before the first is used; keys that are not
+      // seen have weight zero and lie in pages that exist (or in the table's last entry's page)
+      constexpr int PACKS = 64 / PN;
+#pragma unroll
+      for (int c = 0; c < VC; ++c) {
+        const int col = min(lane + 64 * c, value_dim - 1);
+        P16 vv[PACKS];
+#pragma unroll
+        for (int k = 0; k < PACKS; ++k) {
+          const int64_t page = __shfl(my_page, k * PN, DLI_WAVE);
+          vv[k] = *reinterpret_cast<const P16*>(v_pages + ((page * kv_heads + kvh) * value_dim + col) * page_size +
+                                                (j0 + k * PN) % page_size);
+        }
+#pragma unroll
+        for (int k = 0; k < PACKS; ++k)
+#pragma unroll
+          for (int e = 0; e < PN; ++e) {
+            const float vf = to_f32((T)vv[k][e]);
+#pragma unroll
+            for (int h = 0; h < GQ; ++h) acc[h][c] = fmaf(ps[(wave * GQ + h) * 64 + k * PN + e], vf, acc[h][c]);
+          }
+      }
+      __builtin_amdgcn_wave_barrier();
+      continue;
+    }
 #pragma unroll
     for (int c = 0; c < VC; ++c) {
       const int col = lane + 64 * c;
@@ -353,22 +382,22 @@ __global__ __launch_bounds__(256) void attention_scored_decode_kernel(
     const float l = wave_sum(l_run[h]);
     if (lane == 0) {
       ms[wave * GQ + h] = m_run[h];
-      ms[4 * GQ + wave * GQ + h] = l;
+      ms[waves * GQ + wave * GQ + h] = l;
     }
 #pragma unroll
     for (int c = 0; c < VC; ++c) accs[((wave * GQ + h) * VC + c) * 64 + lane] = acc[h][c];
   }
   __syncthreads();
-  for (int idx = tid; idx < nh * value_dim; idx += 256) {
+  for (int idx = tid; idx < nh * value_dim; idx += threads) {
     const int h = idx / value_dim, col = idx - h * value_dim;
     float m = -INFINITY;
-    for (int w = 0; w < 4; ++w) m = fmaxf(m, ms[w * GQ + h]);
+    for (int w = 0; w < waves; ++w) m = fmaxf(m, ms[w * GQ + h]);
     float l = 0.f, o = 0.f;
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < waves; ++w) {
       const float mw = ms[w * GQ + h];
       if (mw > -INFINITY) {
         const float f = expf(mw - m);
-        l += ms[4 * GQ + w * GQ + h] * f;
+        l += ms[waves * GQ + w * GQ + h] * f;
         o += accs[((w * GQ + h) * VC + col / 64) * 64 + col % 64] * f;
       }
     }
@@ -386,10 +415,17 @@ static int launch_scored_decode(const void* q, int64_t q_stride, const void* k_p
                                 int window, ScoreChanges sc, hipStream_t stream) {
   const int group = q_heads / kv_heads, vc = (sc.value_dim + 63) / 64;
   const dim3 grid(entries, kv_heads, (group + GQ - 1) / GQ);
+  // eight waves where their states fit 64 KB of LDS, else four: the chain of a wave's
+  // blocks (table entry, key rows, value rows, each a trip to memory) is as long as its blocks
 #define DECODE_LAUNCH(VC)                                                                                   \
   {                                                                                                         \
-    const size_t bytes = sizeof(float) * ((size_t)GQ * head_dim + 4 * GQ * 64 + 8 * GQ + 4 * GQ * VC * 64); \
-    attention_scored_decode_kernel<T, GQ, VC><<<grid, 256, bytes, stream>>>(                                \
+    int waves = 8;                                                                                          \
+    size_t bytes = 0;                                                                                       \
+    for (;; waves /= 2) {                                                                                   \
+      bytes = sizeof(float) * ((size_t)GQ * head_dim + waves * GQ * 64 + 2 * waves * GQ + waves * GQ * VC * 64); \
+      if (bytes <= 65536 || waves == 4) break;                                                              \
+    }                                                                                                       \
+    attention_scored_decode_kernel<T, GQ, VC><<<grid, 64 * waves, bytes, stream>>>(                         \
         (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, kv_len,           \
         block_tables, table_stride, q_heads, kv_heads, head_dim, page_size, scale, window, sc);             \
   }

@@ -166,8 +166,7 @@ __global__ __launch_bounds__(64) void recurrent_scan_kernel(ScanArgs p) {
   for (int i = 0; i < NK; ++i) st[i] = s[i];
 }
 
-// out = o / sqrt(mean_head(o^2) + eps) * norm_w * gate(g_pre), head by head: one workgroup a row,
-// its waves take the heads in turn.
+// out = o / sqrt(mean_head(o^2) + eps) * norm_w * gate(g_pre), head by head: a wave a (row, head).
 template <typename T, int RULE>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, int64_t o_stride,
                                                              const float* __restrict__ g_pre, int64_t g_stride,
@@ -175,7 +174,8 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
                                                              T* __restrict__ out, int64_t out_stride, int heads, int dim) {
   const int64_t row = blockIdx.x;
   const int lane = threadIdx.x % DLI_WAVE, wave = threadIdx.x / DLI_WAVE;
-  for (int h = wave; h < heads; h += 4) {
+  const int h = blockIdx.y * 4 + wave;
+  if (h < heads) {
     const float* oh = o + row * o_stride + (int64_t)h * dim;
     float ss = 0.f;
     for (int c = lane; c < dim; c += DLI_WAVE) ss += oh[c] * oh[c];
@@ -206,10 +206,10 @@ static int launch_scan(const ScanArgs& p, int entries, int rows, int dim, int ou
 #undef SCAN_CASE
   if (dli_launch_status() != DLI_OK) return DLI_ERR_LAUNCH;
   if (out_is_bf16)
-    head_norm_gate_kernel<bf16_t, RULE><<<rows, 256, 0, stream>>>(p.o_raw, p.o_stride, p.g_pre, p.g_stride, p.norm_w, p.eps,
+    head_norm_gate_kernel<bf16_t, RULE><<<dim3(rows, (p.heads + 3) / 4), 256, 0, stream>>>(p.o_raw, p.o_stride, p.g_pre, p.g_stride, p.norm_w, p.eps,
                                                                   (bf16_t*)p.out, p.out_stride, p.heads, dim);
   else
-    head_norm_gate_kernel<float, RULE><<<rows, 256, 0, stream>>>(p.o_raw, p.o_stride, p.g_pre, p.g_stride, p.norm_w, p.eps,
+    head_norm_gate_kernel<float, RULE><<<dim3(rows, (p.heads + 3) / 4), 256, 0, stream>>>(p.o_raw, p.o_stride, p.g_pre, p.g_stride, p.norm_w, p.eps,
                                                                  (float*)p.out, p.out_stride, p.heads, dim);
   return dli_launch_status();
 }

@@ -85,9 +85,9 @@ __device__ __forceinline__ int entry_of_row(const int* __restrict__ q_start, int
   return lo;
 }
 
-// One workgroup a row. The thread that reads a request's state for the entry's first row is also
-// the one that writes the entry's last row there, after its read: no other thread touches that
-// element in this launch.
+// A thread an element (grid: rows x blocks of the width). The thread that reads a request's state
+// for the entry's first row is also the one that writes the entry's last row there, after its
+// read: no other thread touches that element in this launch.
 template <typename T>
 __global__ void token_shift_kernel(const float* __restrict__ x, const float* __restrict__ mu, int mixes,
                                    float* state, int64_t state_stride, const int* __restrict__ q_start, int entries,
@@ -100,7 +100,8 @@ __global__ void token_shift_kernel(const float* __restrict__ x, const float* __r
   float* st = state + (int64_t)state_slots[e] * state_stride;
   const bool from_state = row == first;
   const bool fresh = positions[row] == 0;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+  const int i = blockIdx.y * blockDim.x + threadIdx.x;
+  if (i < width) {
     const float cur = xr[i];
     float prev;
     if (from_state) {
@@ -249,13 +250,13 @@ int dli_token_shift(const float* x, const float* mu, int mixes, float* state, in
                     int is_bf16, hipStream_t stream) {
   if (rows <= 0) return DLI_OK;
   if (width <= 0 || mixes <= 0 || entries <= 0 || state_stride < width) return DLI_ERR_ARGUMENT;
-  const int threads = width >= 1024 ? 256 : 128;
+  const dim3 grid(rows, (width + 255) / 256);
   if (is_bf16)
-    token_shift_kernel<bf16_t><<<rows, threads, 0, stream>>>(x, mu, mixes, state, state_stride, q_start, entries,
-                                                             positions, state_slots, (bf16_t*)out, rows, width);
+    token_shift_kernel<bf16_t><<<grid, 256, 0, stream>>>(x, mu, mixes, state, state_stride, q_start, entries,
+                                                         positions, state_slots, (bf16_t*)out, rows, width);
   else
-    token_shift_kernel<float><<<rows, threads, 0, stream>>>(x, mu, mixes, state, state_stride, q_start, entries,
-                                                            positions, state_slots, (float*)out, rows, width);
+    token_shift_kernel<float><<<grid, 256, 0, stream>>>(x, mu, mixes, state, state_stride, q_start, entries,
+                                                        positions, state_slots, (float*)out, rows, width);
   return dli_launch_status();
 }
 
