@@ -100,6 +100,10 @@ _SIGNATURES = {
     "dli_attention_scored": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr,
                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_ptr,
                              _c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr],
+    "dli_attention_scored_mfma_supports": [_c_int, _c_int, _c_int],
+    "dli_attention_scored_mfma": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr,
+                                  _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_ptr,
+                                  _c_ptr, _c_ptr, _c_i64, _c_ptr],
     "dli_embed_sinusoid": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "dli_cast_from_f32": [_c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr],
     "dli_norm_into_stream": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr],
@@ -1526,6 +1530,61 @@ def attention_scored(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tens
         _ptr(block_tables), block_tables.stride(0), _ptr(tile_entry), _ptr(tile_q0), tiles, q_heads, kv_heads,
         head_dim, value_dim, page_size, float(scale), int(window), int(chunk), int(bool(sink)), _ptr(r1), _ptr(r2),
         _ptr(gate), gate_stride, _is_bf16(dtype), _stream()), "attention_scored")
+
+
+SCORED_MFMA_TILE_ROWS = 64  # queries of a tile of the matrix-core kernel (four waves of 16)
+
+
+def attention_scored_mfma_supports(head_dim: int, value_dim: int, page_size: int, dtype: torch.dtype) -> bool:
+    return dtype == torch.bfloat16 and bool(
+        library().dli_attention_scored_mfma_supports(int(head_dim), int(value_dim), int(page_size)))
+
+
+def attention_scored_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, out: torch.Tensor,
+                          q_start: torch.Tensor, kv_len: torch.Tensor, block_tables: torch.Tensor,
+                          tile_entry: torch.Tensor, tile_q0: torch.Tensor, q_heads: int, scale: float, *,
+                          window: int = 0, chunk: int = 0, sink: bool = False, r1: Optional[torch.Tensor] = None,
+                          r2: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> None:
+    """:func:`attention_scored` for the portions of a bfloat16 step on the matrix cores: the same
+    operands and parameters, tiles of ``SCORED_MFMA_TILE_ROWS`` queries, sizes that
+    :func:`attention_scored_mfma_supports` takes."""
+    _dense(k_pages, "k_pages", torch.bfloat16, 4)
+    _rows(q, "q", torch.bfloat16)
+    _rows(out, "out", torch.bfloat16)
+    pages, kv_heads, page_size, head_dim = k_pages.shape
+    _dense(v_pages, "v_pages", torch.bfloat16, 4)
+    value_dim = v_pages.shape[2]
+    _require(v_pages.shape == (pages, kv_heads, value_dim, page_size),
+             "v_pages must be [pages, kv_heads, value_dim, page_size]")
+    _require(attention_scored_mfma_supports(head_dim, value_dim, page_size, k_pages.dtype),
+             "the matrix-core kernel does not take these sizes")
+    _require(q.shape[1] == q_heads * head_dim and out.shape == (q.shape[0], q_heads * value_dim),
+             "q must be [tokens, q_heads*head_dim] and out [tokens, q_heads*value_dim]")
+    _require(q_heads % kv_heads == 0, "query heads are not a multiple of kv heads")
+    _require(q.stride(0) % 4 == 0 and out.stride(0) % 4 == 0 and q.data_ptr() % 8 == 0 and out.data_ptr() % 8 == 0,
+             "q and out must be 8-byte aligned, row by row")
+    for name, t in (("q_start", q_start), ("kv_len", kv_len), ("tile_entry", tile_entry), ("tile_q0", tile_q0)):
+        _dense(t, name, torch.int32, 1)
+    _dense(block_tables, "block_tables", torch.int32, 2)
+    entries = kv_len.shape[0]
+    _require(q_start.shape[0] == entries + 1 and block_tables.shape[0] >= entries,
+             "q_start/kv_len/block_tables disagree on the number of requests")
+    _require(tile_entry.shape == tile_q0.shape, "tile lists differ in length")
+    _require((r1 is None) == (r2 is None), "r1 and r2 come together")
+    for name, t in (("r1", r1), ("r2", r2)):
+        if t is not None:
+            _dense(t, name, torch.float32, 1)
+            _require(t.shape[0] == q_heads, f"{name} must hold one value per query head")
+    gate_stride = 0
+    if gate is not None:
+        _f32_rows(gate, "gate")
+        _require(gate.shape == out.shape, "gate differs from out in shape")
+        gate_stride = gate.stride(0)
+    _check(library().dli_attention_scored_mfma(
+        _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(q_start), _ptr(kv_len),
+        _ptr(block_tables), block_tables.stride(0), _ptr(tile_entry), _ptr(tile_q0), tile_entry.shape[0], q_heads,
+        kv_heads, head_dim, value_dim, page_size, float(scale), int(window), int(chunk), int(bool(sink)), _ptr(r1),
+        _ptr(r2), _ptr(gate), gate_stride, _stream()), "attention_scored_mfma")
 
 
 RULE_DELTA, RULE_BONUS = 0, 1

@@ -134,11 +134,23 @@ class ScoredAttention(Mixer):
                           v_first_in=first_in, v_first_out=first_out)
         out = self.rt.empty(n, self._o)
         gate = proj[:, self._q + self._k + self._v:] if self.output_gate else None
-        if ctx.num_decode == ctx.num_entries:
-            tiles = (None, None)  # every entry is one row: nothing is derived from the step's lengths on the host
+        changes = dict(window=self.window, chunk=self.chunk, sink=self.sink, r1=self.r1, r2=self.r2)
+        nd = ctx.num_decode
+        if nd == ctx.num_entries:
+            # every entry is one row: nothing is derived from the step's lengths on the host
+            ops.attention_scored(q, cache.k_pages, cache.v_pages, out, ctx.q_start, ctx.kv_len, grp.block_tables,
+                                 None, None, self.num_heads, self.scale, gate=gate, **changes)
+        elif ops.attention_scored_mfma_supports(self.head_dim, self.value_dim, ctx.page_size, self.rt.dtype):
+            # single tokens (they come first) to their kernel, portions to the matrix cores
+            if nd:
+                ops.attention_scored(q[:nd], cache.k_pages, cache.v_pages, out[:nd], ctx.q_start[:nd + 1], ctx.kv_len[:nd],
+                                     grp.block_tables[:nd], None, None, self.num_heads, self.scale,
+                                     gate=None if gate is None else gate[:nd], **changes)
+            tiles = ctx.q_tiles(ops.SCORED_MFMA_TILE_ROWS, first_entry=nd)
+            ops.attention_scored_mfma(q, cache.k_pages, cache.v_pages, out, ctx.q_start, ctx.kv_len, grp.block_tables,
+                                      tiles[0], tiles[1], self.num_heads, self.scale, gate=gate, **changes)
         else:
             tiles = ctx.q_tiles(ops.attention_generic_tile_rows(max(self.head_dim, self.value_dim)))
-        ops.attention_scored(q, cache.k_pages, cache.v_pages, out, ctx.q_start, ctx.kv_len, grp.block_tables,
-                             tiles[0], tiles[1], self.num_heads, self.scale, window=self.window, chunk=self.chunk,
-                             sink=self.sink, r1=self.r1, r2=self.r2, gate=gate)
+            ops.attention_scored(q, cache.k_pages, cache.v_pages, out, ctx.q_start, ctx.kv_len, grp.block_tables,
+                                 tiles[0], tiles[1], self.num_heads, self.scale, gate=gate, **changes)
         return linear_f32(self.rt, out, self.w_o)

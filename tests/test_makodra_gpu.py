@@ -129,20 +129,23 @@ def paged(k, v, page_size, dtype, seed=0, spare=3):
     return kp, vp, order[:pages]
 
 
-def run_attention(ops, q, kp, vp, table, q_rows, n_keys, heads, scale, *, decode=False, gate=None, **changes):
-    """The last ``q_rows`` queries of a request of ``n_keys`` keys; ``decode``: without tile lists."""
+def run_attention(ops, q, kp, vp, table, q_rows, n_keys, heads, scale, *, decode=False, gate=None, mfma=False,
+                  **changes):
+    """The last ``q_rows`` queries of a request of ``n_keys`` keys; ``decode``: without tile lists;
+    ``mfma``: the matrix-core kernel for portions."""
     dtype = kp.dtype
     V = vp.shape[2]
     out = torch.zeros(q_rows, heads * V, dtype=dtype).cuda()
     if decode:
         tiles = (None, None)
     else:
-        rows = ops.attention_generic_tile_rows(max(kp.shape[3], V))
+        rows = ops.SCORED_MFMA_TILE_ROWS if mfma else ops.attention_generic_tile_rows(max(kp.shape[3], V))
         q0s = list(range(0, q_rows, rows))
         tiles = (i32([0] * len(q0s)), i32(q0s))
-    ops.attention_scored(q.to(dtype).cuda(), kp.cuda(), vp.cuda(), out, i32([0, q_rows]), i32([n_keys]),
-                         i32(table).view(1, -1), tiles[0], tiles[1], heads, scale,
-                         gate=None if gate is None else gate.float().cuda(), **changes)
+    kernel = ops.attention_scored_mfma if mfma else ops.attention_scored
+    kernel(q.to(dtype).cuda(), kp.cuda(), vp.cuda(), out, i32([0, q_rows]), i32([n_keys]),
+           i32(table).view(1, -1), tiles[0], tiles[1], heads, scale,
+           gate=None if gate is None else gate.float().cuda(), **changes)
     return out.cpu().double()
 
 
@@ -168,14 +171,21 @@ def test_attention_with_every_change_of_the_scores(ops, dtype, H, G, D, V, ps):
         dev_case = {n_: (t.cuda() if isinstance(t, torch.Tensor) else t) for n_, t in case.items()}
         got = run_attention(ops, q.reshape(n, H * D), kp, vp, table, n, n, H, 0.7, **dev_case)
         assert (got - ref.reshape(n, H * V)).abs().max() < tol, case
-        # the same rows as portions on top of cached keys, down to one row without tile lists, and gated
-        for first in (n - 1, n - 2, 40):
+        matrix_cores = ops.attention_scored_mfma_supports(D, V, ps, dtype)
+        assert matrix_cores == (dtype == torch.bfloat16 and D % 16 == 0 and V % 16 == 0 and ps % 4 == 0)
+        # the same rows as portions on top of cached keys, down to one row without tile lists, and gated;
+        # portions also through the matrix-core kernel where it takes the sizes
+        for first in (n - 1, n - 2, 40, 0):
             rows = n - first
             g = gate[first:]
+            want = ref[first:].reshape(rows, H * V) * torch.sigmoid(g.double())
             got = run_attention(ops, q[first:].reshape(rows, H * D), kp, vp, table, rows, n, H, 0.7,
                                 decode=rows == 1, gate=g, **dev_case)
-            want = ref[first:].reshape(rows, H * V) * torch.sigmoid(g.double())
             assert (got - want).abs().max() < tol, (case, first)
+            if matrix_cores:
+                got = run_attention(ops, q[first:].reshape(rows, H * D), kp, vp, table, rows, n, H, 0.7, gate=g, mfma=True,
+                                    **dev_case)
+                assert (got - want).abs().max() < tol, (case, first, "matrix cores")
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -208,6 +218,10 @@ def test_attention_sees_a_planted_key_inside_its_chunk_only(ops, dtype):
             got = run_attention(ops, q[first:query + 1].reshape(rows, H * D), kp, vp, table, rows, query + 1, H, 1.0,
                                 decode=rows == 1, chunk=chunk, sink=True)
             assert (got - ref[first:query + 1].reshape(rows, H * V)).abs().max() < tol, (planted, query, first)
+            if dtype == torch.bfloat16:
+                got = run_attention(ops, q[first:query + 1].reshape(rows, H * D), kp, vp, table, rows, query + 1, H, 1.0,
+                                    mfma=True, chunk=chunk, sink=True)
+                assert (got - ref[first:query + 1].reshape(rows, H * V)).abs().max() < tol, (planted, query, first, "matrix cores")
 
 
 def test_unit_queries_and_keys_value_mix_and_cache_write(ops):
