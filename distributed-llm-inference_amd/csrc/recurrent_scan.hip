@@ -1,20 +1,25 @@
 // Linear recurrences with a matrix state per head, S [key channel][value channel] in 32-bit,
 // carried from token to token of a request in its state slot. Two rules, one kernel:
 //
-//   RULE_DELTA   u = k / sqrt(sum k^2 + 1e-6);  w = exp(-exp(-1/2) sigmoid(w_pre));  a = sigmoid(a_pre + a_bias)
+//   RULE_DELTA   u = k / sqrt(sum k^2 + 1e-6);
 //                S <- diag(w) S - (a * u) (u^T S) + k v^T   (both terms read the old S);   o = S^T r
-//   RULE_BONUS   w = exp(-exp(w_pre));   o = (S + diag(bonus) k v^T)^T r;   S <- diag(w) S + k v^T
+//   RULE_BONUS   o = (S + diag(bonus) k v^T)^T r;   S <- diag(w) S + k v^T
+//
+// with the decay w and the removal rate a per key channel given ready made (32-bit; the kernel of
+// the low-rank projection's second half makes them: every wave of a head would otherwise repeat
+// their exponentials),
 //
 // followed, per token and head, by o / sqrt(mean(o^2) + eps) * norm_w * gate, with gate =
 // sigmoid(g_pre) (RULE_DELTA) or silu(g_pre) (RULE_BONUS); the result is written in the type of
 // the product that reads it. Everything here is 32-bit arithmetic on 32-bit inputs.
 //
-// One wave takes one (entry, head, slice of 8 value columns) and walks the entry's tokens in
-// order; waves never wait for each other. Lane (v, part) keeps the D / 8 state values
-// S[part's keys][v] in registers: a column of S never leaves its eight neighbouring lanes, whose
-// partial dot products meet in three DPP swaps. A wave alone on its SIMD issues an instruction
+// One wave takes one (entry, head, slice of 4 value columns) and walks the entry's tokens in
+// order; waves never wait for each other. Lane (v, part) keeps the D / 16 state values
+// S[part's keys][v] in registers: a column of S never leaves its sixteen neighbouring lanes (a DPP
+// row), whose partial dot products meet in four DPP swaps (heads whose size is no multiple of 16:
+// eight lanes a column, eight columns a wave). A wave alone on its SIMD issues an instruction
 // every four to five cycles, so the chain over a request's tokens is as long as a token's
-// instructions: eight lanes a column keep that to some hundred. The per-token vectors of 16
+// instructions: many lanes a column keep that to some fifty. The per-token vectors of 16
 // tokens (8 for heads above 64; one in a step of single tokens) are staged in LDS at once: the
 // loads of the next batch are in flight while the chain over this batch's tokens runs, and the
 // chain itself reads LDS and registers only. o goes out in 32-bit; a second kernel normalises
@@ -31,8 +36,8 @@
 
 struct ScanArgs {
   const float* r; const float* k; const float* v;   // [rows][heads * D], each with its row stride
-  const float* w_pre;                                // decay before its activation
-  const float* a_pre; const float* a_bias;           // RULE_DELTA: removal rate before the sigmoid, its bias [heads * D]
+  const float* w_pre;                                // the decay w
+  const float* a_pre; const float* a_bias;           // RULE_DELTA: the removal rate a (a_bias is not read)
   const float* g_pre;                                // gate before its activation
   int64_t r_stride, k_stride, v_stride, w_stride, a_stride, g_stride;
   const float* bonus;                                // RULE_BONUS: [heads][D]
@@ -54,12 +59,21 @@ __device__ __forceinline__ float octet_sum(float x) {
   return x;
 }
 
-template <int NK, int RULE, int TB>
+// Sum over the sixteen lanes of a row: the octet's sum, then the mirror of the row, which swaps its octets.
+__device__ __forceinline__ float row_sum(float x) {
+  x = octet_sum(x);
+  x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x140, 0xF, 0xF, false));
+  return x;
+}
+template <int PARTS> __device__ __forceinline__ float parts_sum(float x) { return PARTS == 16 ? row_sum(x) : octet_sum(x); }
+
+// PARTS lanes share a value column (16 where the head's size allows, else 8); a wave holds 64 / PARTS columns.
+template <int NK, int PARTS, int RULE, int TB>
 __global__ __launch_bounds__(64) void recurrent_scan_kernel(ScanArgs p) {
-  constexpr int D = NK * 8, PER = (TB * D + 63) / 64;  // PER: what a lane stages per vector and batch
+  constexpr int D = NK * PARTS, COLS = 64 / PARTS, PER = (TB * D + 63) / 64;  // PER: what a lane stages per vector and batch
   __shared__ float sk[PER * 64], sw[PER * 64], sa[RULE == RULE_DELTA ? PER * 64 : 1], sr[PER * 64];
-  const int lane = threadIdx.x, vloc = lane >> 3, part = lane & 7;
-  const int entry = blockIdx.x, head = blockIdx.y, col = blockIdx.z * 8 + vloc;
+  const int lane = threadIdx.x, vloc = lane / PARTS, part = lane % PARTS;
+  const int entry = blockIdx.x, head = blockIdx.y, col = blockIdx.z * COLS + vloc;
   const int row0 = p.q_start[entry], n_rows = p.q_start[entry + 1] - row0;
   if (n_rows <= 0) return;
   const int64_t col0 = (int64_t)head * D;
@@ -72,7 +86,7 @@ __global__ __launch_bounds__(64) void recurrent_scan_kernel(ScanArgs p) {
     bon[i] = RULE == RULE_BONUS ? p.bonus[col0 + part * NK + i] : 0.f;
   }
 
-  constexpr int PV = (TB * 8 + 63) / 64;
+  constexpr int PV = (TB * COLS + 63) / 64;
   __shared__ float sv[PV * 64], skn[TB];
   float pk[PER], pw[PER], pa[PER], pr[PER], pv[PV];
   auto fetch = [&](int t0) {
@@ -83,12 +97,12 @@ __global__ __launch_bounds__(64) void recurrent_scan_kernel(ScanArgs p) {
       pk[m] = p.k[row * p.k_stride + col0 + c];
       pr[m] = p.r[row * p.r_stride + col0 + c];
       pw[m] = p.w_pre[row * p.w_stride + col0 + c];
-      if (RULE == RULE_DELTA) pa[m] = p.a_pre[row * p.a_stride + col0 + c] + p.a_bias[col0 + c];
+      if (RULE == RULE_DELTA) pa[m] = p.a_pre[row * p.a_stride + col0 + c];
     }
 #pragma unroll
     for (int m = 0; m < PV; ++m) {
-      const int e = min(lane + 64 * m, TB * 8 - 1);
-      pv[m] = p.v[(int64_t)(row0 + min(t0 + e / 8, n_rows - 1)) * p.v_stride + col0 + blockIdx.z * 8 + e % 8];
+      const int e = min(lane + 64 * m, TB * COLS - 1);
+      pv[m] = p.v[(int64_t)(row0 + min(t0 + e / COLS, n_rows - 1)) * p.v_stride + col0 + blockIdx.z * COLS + e % COLS];
     }
   };
   // One token of the chain, from LDS and registers only. Nothing but s hangs on the token before:
@@ -97,20 +111,20 @@ __global__ __launch_bounds__(64) void recurrent_scan_kernel(ScanArgs p) {
     const float* kt = sk + t * D + part * NK;
     const float* wt = sw + t * D + part * NK;
     const float* rt = sr + t * D + part * NK;
-    const float v = sv[t * 8 + vloc];
+    const float v = sv[t * COLS + vloc];
     float o0 = 0.f, o1 = 0.f;
     if (RULE == RULE_DELTA) {
-      const float* at = sa + t * D + part * NK;
+      const float* at = sa + t * D + part * NK;     // a * u, made when the batch was staged
       const float kn = skn[t];
       float ks0 = 0.f, ks1 = 0.f;
 #pragma unroll
       for (int i = 0; i < NK; ++i) {
         if (i & 1) ks1 = fmaf(kt[i], s[i], ks1); else ks0 = fmaf(kt[i], s[i], ks0);
       }
-      const float us = octet_sum(ks0 + ks1) * kn;       // u^T S for this column, u = k * kn
+      const float us = parts_sum<PARTS>(ks0 + ks1) * kn;       // u^T S for this column, u = k * kn
 #pragma unroll
       for (int i = 0; i < NK; ++i) {
-        s[i] = wt[i] * s[i] - (at[i] * (kt[i] * kn)) * us + kt[i] * v;
+        s[i] = wt[i] * s[i] - at[i] * us + kt[i] * v;
         if (i & 1) o1 = fmaf(s[i], rt[i], o1); else o0 = fmaf(s[i], rt[i], o0);
       }
     } else {
@@ -121,7 +135,7 @@ __global__ __launch_bounds__(64) void recurrent_scan_kernel(ScanArgs p) {
         s[i] = wt[i] * s[i] + kv;
       }
     }
-    const float o = octet_sum(o0 + o1);
+    const float o = parts_sum<PARTS>(o0 + o1);
     if (part == 0) p.o_raw[row * p.o_stride + col0 + col] = o;
   };
   fetch(0);
@@ -131,12 +145,8 @@ __global__ __launch_bounds__(64) void recurrent_scan_kernel(ScanArgs p) {
       const int e = lane + 64 * m;
       sk[e] = pk[m];
       sr[e] = pr[m];
-      if (RULE == RULE_DELTA) {
-        sw[e] = expf(-0.6065306597126334f / (1.f + expf(-pw[m])));
-        sa[e] = 1.f / (1.f + expf(-pa[m]));
-      } else {
-        sw[e] = expf(-expf(pw[m]));
-      }
+      sw[e] = pw[m];
+      if (RULE == RULE_DELTA) sa[e] = pa[m];
     }
 #pragma unroll
     for (int m = 0; m < PV; ++m) sv[lane + 64 * m] = pv[m];
@@ -150,6 +160,13 @@ __global__ __launch_bounds__(64) void recurrent_scan_kernel(ScanArgs p) {
         kk += __shfl_xor(kk, 1, DLI_WAVE);
         kk += __shfl_xor(kk, 2, DLI_WAVE);
         if ((lane & 3) == 0) skn[t] = 1.f / sqrtf(kk + 1e-6f);
+      }
+      __syncthreads();
+      // the removal rate times the unit key, a * u = a * k / |k|, off the chain as well
+#pragma unroll
+      for (int m = 0; m < PER; ++m) {
+        const int e = lane + 64 * m;
+        sa[e] *= sk[e] * skn[min(e / D, TB - 1)];
       }
       __syncthreads();
     }
@@ -190,17 +207,20 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
 
 template <int RULE>
 static int launch_scan(const ScanArgs& p, int entries, int rows, int dim, int out_is_bf16, hipStream_t stream) {
-  const dim3 grid(entries, p.heads, dim / 8);
+  // sixteen lanes a column (four columns a wave) where the head's size is a multiple of 16, else eight
+  const int parts = dim % 16 == 0 ? 16 : 8;
+  const dim3 grid(entries, p.heads, dim / (64 / parts));
   // a step of single tokens stages one token a wave; any other stages 16 (8 for heads above 64)
   const bool single = rows == entries;
-#define SCAN_CASE(NK, TBM)                                                                           \
-  case NK:                                                                                           \
-    if (single) recurrent_scan_kernel<NK, RULE, 1><<<grid, 64, 0, stream>>>(p);                      \
-    else recurrent_scan_kernel<NK, RULE, TBM><<<grid, 64, 0, stream>>>(p);                           \
+#define SCAN_CASE(DIM, PARTS, TBM)                                                                          \
+  case DIM:                                                                                                 \
+    if (single) recurrent_scan_kernel<DIM / PARTS, PARTS, RULE, 1><<<grid, 64, 0, stream>>>(p);             \
+    else recurrent_scan_kernel<DIM / PARTS, PARTS, RULE, TBM><<<grid, 64, 0, stream>>>(p);                  \
     break;
-  switch (dim / 8) {
-    SCAN_CASE(2, 16) SCAN_CASE(3, 16) SCAN_CASE(4, 16) SCAN_CASE(5, 16) SCAN_CASE(6, 16) SCAN_CASE(7, 16)
-    SCAN_CASE(8, 16) SCAN_CASE(10, 8) SCAN_CASE(12, 8) SCAN_CASE(14, 8) SCAN_CASE(16, 8)
+  switch (dim) {
+    SCAN_CASE(16, 16, 16) SCAN_CASE(24, 8, 16) SCAN_CASE(32, 16, 16) SCAN_CASE(40, 8, 16) SCAN_CASE(48, 16, 16)
+    SCAN_CASE(56, 8, 16) SCAN_CASE(64, 16, 16) SCAN_CASE(80, 16, 8) SCAN_CASE(96, 16, 8) SCAN_CASE(112, 16, 8)
+    SCAN_CASE(128, 16, 8)
     default: return DLI_ERR_ARGUMENT;
   }
 #undef SCAN_CASE
@@ -230,7 +250,7 @@ extern "C" int dli_recurrent_scan(const float* r, int64_t r_stride, const float*
                                   int out_is_bf16, hipStream_t stream) {
   if (entries <= 0 || rows <= 0) return DLI_OK;
   if (rows < entries || !dli_recurrent_scan_supports(dim) || heads <= 0 || heads > 65535 || (rule != RULE_DELTA && rule != RULE_BONUS) ||
-      state_stride < (int64_t)heads * dim * dim || (rule == RULE_DELTA && (a_pre == nullptr || a_bias == nullptr)) ||
+      state_stride < (int64_t)heads * dim * dim || (rule == RULE_DELTA && a_pre == nullptr) ||
       (rule == RULE_BONUS && bonus == nullptr))
     return DLI_ERR_ARGUMENT;
   ScanArgs p;

@@ -117,9 +117,14 @@ __global__ void token_shift_kernel(const float* __restrict__ x, const float* __r
 
 // act: 0 none, 1 tanh. t is [rows][t_stride] (rank values a row), w2t [rank][features] (the matrix
 // transposed, so that neighbouring threads read neighbouring weights), out [rows][features].
+// out_act: what becomes of y before it is stored: 0 y itself; 1 exp(-exp(-1/2) sigmoid(y)) and
+// 2 exp(-exp(y)), the decays of the two recurrences. rate (may be nullptr): [rows][rate_stride], with
+// features values a row that become sigmoid(rate + rate_bias) in place (the delta rule's removal
+// rate, made here because a thread a (row, feature) is what this launch already has).
 __global__ void lowrank_out_kernel(const float* __restrict__ t, int64_t t_stride, const float* __restrict__ w2t,
                                    const float* __restrict__ bias, float* __restrict__ out, int features, int rank,
-                                   int act) {
+                                   int act, int out_act, float* __restrict__ rate, int64_t rate_stride,
+                                   const float* __restrict__ rate_bias) {
   extern __shared__ float ts[];
   const int64_t row = blockIdx.x;
   for (int j = threadIdx.x; j < rank; j += blockDim.x) {
@@ -140,7 +145,14 @@ __global__ void lowrank_out_kernel(const float* __restrict__ t, int64_t t_stride
     s3 = fmaf(ts[j + 3], e, s3);
   }
   for (; j < rank; ++j) s0 = fmaf(ts[j], w2t[(int64_t)j * features + c], s0);
-  out[row * features + c] = ((s0 + s1) + (s2 + s3)) + (bias != nullptr ? bias[c] : 0.f);
+  float y = ((s0 + s1) + (s2 + s3)) + (bias != nullptr ? bias[c] : 0.f);
+  if (out_act == 1) y = expf(-0.6065306597126334f / (1.f + expf(-y)));
+  else if (out_act == 2) y = expf(-expf(y));
+  out[row * features + c] = y;
+  if (rate != nullptr) {
+    float* r = rate + row * rate_stride + c;
+    *r = 1.f / (1.f + expf(-(*r + (rate_bias != nullptr ? rate_bias[c] : 0.f))));
+  }
 }
 
 // proj [tokens][stride] float32 holds q (q_heads x dim), k (kv_heads x dim) and v (kv_heads x vdim)
@@ -261,11 +273,15 @@ int dli_token_shift(const float* x, const float* mu, int mixes, float* state, in
 }
 
 int dli_lowrank_out(const float* t, int64_t t_stride, const float* w2t, const float* bias, float* out, int rows,
-                    int features, int rank, int act, hipStream_t stream) {
+                    int features, int rank, int act, int out_act, float* rate, int64_t rate_stride,
+                    const float* rate_bias, hipStream_t stream) {
   if (rows <= 0) return DLI_OK;
-  if (features <= 0 || rank <= 0 || rank > 8192 || t_stride < rank || act < 0 || act > 1) return DLI_ERR_ARGUMENT;
+  if (features <= 0 || rank <= 0 || rank > 8192 || t_stride < rank || act < 0 || act > 1 || out_act < 0 || out_act > 2 ||
+      (rate != nullptr && rate_stride < features))
+    return DLI_ERR_ARGUMENT;
   lowrank_out_kernel<<<dim3(rows, (features + 255) / 256), 256, rank * sizeof(float), stream>>>(t, t_stride, w2t, bias, out,
-                                                                                                features, rank, act);
+                                                                                                features, rank, act, out_act,
+                                                                                                rate, rate_stride, rate_bias);
   return dli_launch_status();
 }
 

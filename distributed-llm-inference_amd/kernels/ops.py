@@ -111,7 +111,8 @@ _SIGNATURES = {
     "dli_softcap": [_c_ptr, _c_i64, _c_float, _c_ptr],
     "dli_token_shift": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
                         _c_int, _c_ptr],
-    "dli_lowrank_out": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_lowrank_out": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_i64,
+                        _c_ptr, _c_ptr],
     "dli_qk_unit_cache": [_c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                           _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "dli_recurrent_scan_supports": [_c_int],
@@ -1423,11 +1424,18 @@ def token_shift(x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, q_start:
                                      _is_bf16(out.dtype), _stream()), "token_shift")
 
 
+LOWRANK_OUT_ACTS = {"none": 0, "delta_decay": 1, "double_exp_decay": 2}
+
+
 def lowrank_out(t: torch.Tensor, w2t: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
-                act: str = "tanh") -> None:
-    """``out = act(t) @ w2t + bias`` in 32-bit: ``t`` float32 ``[n, rank]`` (rows contiguous, any row
-    stride), ``w2t`` float32 ``[rank, features]`` (the projection's second matrix transposed);
-    ``act`` ``"tanh"`` or ``"none"``."""
+                act: str = "tanh", out_act: str = "none", rate: Optional[torch.Tensor] = None,
+                rate_bias: Optional[torch.Tensor] = None) -> None:
+    """``out = out_act(act(t) @ w2t + bias)`` in 32-bit: ``t`` float32 ``[n, rank]`` (rows contiguous, any
+    row stride), ``w2t`` float32 ``[rank, features]`` (the projection's second matrix transposed);
+    ``act`` ``"tanh"`` or ``"none"``; ``out_act`` ``"none"``, ``"delta_decay"`` (``exp(-exp(-1/2) sigmoid(y))``)
+    or ``"double_exp_decay"`` (``exp(-exp(y))``). ``rate`` (float32 ``[n, features]``, rows contiguous)
+    becomes ``sigmoid(rate + rate_bias)`` in place in the same launch."""
+    _require(out_act in LOWRANK_OUT_ACTS, f"out_act must be one of {sorted(LOWRANK_OUT_ACTS)}")
     _f32_rows(t, "t")
     _dense(w2t, "w2t", torch.float32, 2)
     _dense(out, "out", torch.float32, 2)
@@ -1438,8 +1446,17 @@ def lowrank_out(t: torch.Tensor, w2t: torch.Tensor, bias: Optional[torch.Tensor]
     if bias is not None:
         _dense(bias, "bias", torch.float32, 1)
         _require(bias.shape[0] == feats, "bias length differs from the features")
+    rate_stride = 0
+    if rate is not None:
+        _f32_rows(rate, "rate")
+        _require(rate.shape == (n, feats), "rate must be [n, features]")
+        rate_stride = rate.stride(0)
+        if rate_bias is not None:
+            _dense(rate_bias, "rate_bias", torch.float32, 1)
+            _require(rate_bias.shape[0] == feats, "rate_bias length differs from the features")
     _check(library().dli_lowrank_out(_ptr(t), t.stride(0), _ptr(w2t), _ptr(bias), _ptr(out), n, feats, rank,
-                                     1 if act == "tanh" else 0, _stream()), "lowrank_out")
+                                     1 if act == "tanh" else 0, LOWRANK_OUT_ACTS[out_act], _ptr(rate), rate_stride,
+                                     _ptr(rate_bias), _stream()), "lowrank_out")
 
 
 def qk_unit_cache(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, q_out: torch.Tensor,
@@ -1594,18 +1611,18 @@ def recurrent_scan_supports(dim: int) -> bool:
     return bool(library().dli_recurrent_scan_supports(int(dim)))
 
 
-def recurrent_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, w_pre: torch.Tensor, g_pre: torch.Tensor,
+def recurrent_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, w: torch.Tensor, g_pre: torch.Tensor,
                    norm_w: torch.Tensor, eps: float, state: torch.Tensor, q_start: torch.Tensor,
                    positions: torch.Tensor, state_slots: torch.Tensor, out: torch.Tensor, heads: int, dim: int,
-                   rule: int, a_pre: Optional[torch.Tensor] = None, a_bias: Optional[torch.Tensor] = None,
-                   bonus: Optional[torch.Tensor] = None) -> None:
+                   rule: int, a: Optional[torch.Tensor] = None, bonus: Optional[torch.Tensor] = None) -> None:
     """A matrix-state recurrence per request and head, with the per-head norm and the gate of its
-    output (``csrc/recurrent_scan.hip`` states both rules). ``r, k, v, w_pre, g_pre, a_pre`` are
-    float32 ``[n, heads*dim]`` with contiguous rows (any row stride); ``state`` is float32
-    ``[slots, >= heads*dim*dim]``, row ``state_slots[e]`` being entry ``e``'s; ``out [n, heads*dim]``
-    float32 or bfloat16."""
+    output (``csrc/recurrent_scan.hip`` states both rules). ``r, k, v``, the decay ``w``, the gate's
+    pre-activation ``g_pre`` and (delta rule) the removal rate ``a`` are float32 ``[n, heads*dim]`` with
+    contiguous rows (any row stride); ``state`` is float32 ``[slots, >= heads*dim*dim]``, row
+    ``state_slots[e]`` being entry ``e``'s; ``out [n, heads*dim]`` float32 or bfloat16."""
     n, width = out.shape[0], heads * dim
-    for name, t in (("r", r), ("k", k), ("v", v), ("w_pre", w_pre), ("g_pre", g_pre), ("a_pre", a_pre)):
+    w_pre, a_pre, a_bias = w, a, None
+    for name, t in (("r", r), ("k", k), ("v", v), ("w", w), ("g_pre", g_pre), ("a", a)):
         if t is not None:
             _f32_rows(t, name)
             _require(t.shape == (n, width), f"{name} must be [n, heads*dim]")
@@ -1621,9 +1638,7 @@ def recurrent_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, w_pre: tor
     entries = state_slots.shape[0]
     _require(q_start.shape[0] == entries + 1 and positions.shape[0] == n, "q_start/state_slots/positions disagree")
     if rule == RULE_DELTA:
-        _require(a_pre is not None and a_bias is not None, "the delta rule needs a_pre and a_bias")
-        _dense(a_bias, "a_bias", torch.float32, 1)
-        _require(a_bias.shape[0] == width, "a_bias must hold heads*dim values")
+        _require(a is not None, "the delta rule needs the removal rate")
     else:
         _require(rule == RULE_BONUS and bonus is not None, "the bonus rule needs bonus")
         _dense(bonus, "bonus", torch.float32)

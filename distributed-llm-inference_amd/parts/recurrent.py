@@ -98,11 +98,13 @@ class GeneralDelta(_MatrixStateMixer):
         n, c = x.shape[0], self.width
         proj = linear_f32(self.rt, as_operand(self.rt, x, ctx), self.w_in)
         r, k, v, g, a = (proj[:, i * c:(i + 1) * c] for i in range(5))
-        w_pre = torch.empty(n, c, device=self.rt.device, dtype=torch.float32)
-        ops.lowrank_out(proj[:, 5 * c:5 * c + self.rank], self.w2t, self.w0, w_pre, act="tanh")
+        # the decay, and in the same launch the removal rate in place: sigmoid(W_a h + b_a)
+        w = torch.empty(n, c, device=self.rt.device, dtype=torch.float32)
+        ops.lowrank_out(proj[:, 5 * c:5 * c + self.rank], self.w2t, self.w0, w, act="tanh", out_act="delta_decay",
+                        rate=a, rate_bias=self.a_bias)
         out = self.rt.empty(n, c)
-        ops.recurrent_scan(r, k, v, w_pre, g, self.norm_w, self.norm_eps, state, ctx.q_start, ctx.positions,
-                           ctx.state_slots, out, self.num_heads, self.head_dim, self.rule, a_pre=a, a_bias=self.a_bias)
+        ops.recurrent_scan(r, k, v, w, g, self.norm_w, self.norm_eps, state, ctx.q_start, ctx.positions,
+                           ctx.state_slots, out, self.num_heads, self.head_dim, self.rule, a=a)
         return linear_f32(self.rt, out, self.w_o)
 
 
@@ -149,9 +151,9 @@ class WKV(_MatrixStateMixer):
             linear_f32(self.rt, mixes[i], self.w[name], out=proj[:, i * c:(i + 1) * c])
         linear_f32(self.rt, mixes[4], self.w1, out=proj[:, 4 * c:4 * c + self.rank])
         r, k, v, g = (proj[:, i * c:(i + 1) * c] for i in range(4))
-        w_pre = torch.empty(n, c, device=self.rt.device, dtype=torch.float32)
-        ops.lowrank_out(proj[:, 4 * c:4 * c + self.rank], self.w2t, self.w0, w_pre, act="tanh")
+        w = torch.empty(n, c, device=self.rt.device, dtype=torch.float32)
+        ops.lowrank_out(proj[:, 4 * c:4 * c + self.rank], self.w2t, self.w0, w, act="tanh", out_act="double_exp_decay")
         out = self.rt.empty(n, c)
-        ops.recurrent_scan(r, k, v, w_pre, g, self.norm_w, self.norm_eps, state[:, h:], ctx.q_start, ctx.positions,
+        ops.recurrent_scan(r, k, v, w, g, self.norm_w, self.norm_eps, state[:, h:], ctx.q_start, ctx.positions,
                            ctx.state_slots, out, self.num_heads, self.head_dim, self.rule, bonus=self.bonus)
         return linear_f32(self.rt, out, self.w_o)

@@ -296,8 +296,14 @@ def test_recurrence_in_steps_against_whole(ops, rule, H, D):
         out = torch.empty(rows, c).cuda()
         q_start = np.cumsum([0] + [n for _, n in step])
         positions = [p for name, n in step for p in range(at[name], at[name] + n)]
-        kw = dict(a_pre=pick("a"), a_bias=a_bias.cuda()) if rule == "delta" else dict(bonus=bonus.cuda())
-        ops.recurrent_scan(pick("r"), pick("k"), pick("v"), pick("w"), pick("g"), norm_w.cuda(), eps, state, i32(q_start),
+        # the decay and the rate come ready made, from the kernel that ends the low-rank projection
+        feats = pick("w")
+        decay, rate = torch.empty_like(feats), pick("a")
+        eye = torch.eye(c).cuda()
+        ops.lowrank_out(feats, eye, None, decay, act="none", out_act="delta_decay" if rule == "delta" else "double_exp_decay",
+                        rate=rate if rule == "delta" else None, rate_bias=a_bias.cuda() if rule == "delta" else None)
+        kw = dict(a=rate) if rule == "delta" else dict(bonus=bonus.cuda())
+        ops.recurrent_scan(pick("r"), pick("k"), pick("v"), decay, pick("g"), norm_w.cuda(), eps, state, i32(q_start),
                            i32(positions), i32([slot[name] for name, _ in step]), out, H, D,
                            ops.RULE_DELTA if rule == "delta" else ops.RULE_BONUS, **kw)
         o = out.cpu().double()
