@@ -59,7 +59,9 @@ class MakodraLayer:
             kv = _positive(m.get("kv_heads") or heads, where + ".mixer.kv_heads")
             if heads % kv:
                 raise UnsupportedModelError(f"{where}: {heads} heads do not group onto {kv} kv_heads")
-            mask = m.get("mask") or {}
+            mask = dict(m.get("mask") or {})
+            if str(mask.pop("kind", "chunk")).lower() not in ("chunk", "chunked"):
+                raise UnsupportedModelError(f"{where}.mixer.mask.kind={m['mask']['kind']!r}; known: 'chunk'")
             unknown = set(mask) - {"size"}
             if unknown:
                 raise UnsupportedModelError(f"{where}.mixer.mask has keys that are not implemented: {sorted(unknown)}")

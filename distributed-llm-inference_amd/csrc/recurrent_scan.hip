@@ -183,6 +183,56 @@ __global__ __launch_bounds__(64) void recurrent_scan_kernel(ScanArgs p) {
   for (int i = 0; i < NK; ++i) st[i] = s[i];
 }
 
+// Heads of any other size (1 to 1024): a thread a value column, the column's state read and written in
+// the request's slot token by token, the token's vectors in LDS. Slow, and only there so that no
+// size is refused; the same sums in the same order per column as above are not promised, the same
+// result to rounding is.
+template <int RULE>
+__global__ void recurrent_scan_any_kernel(ScanArgs p, int D) {
+  extern __shared__ float sh[];
+  float *sk = sh, *sw = sh + D, *sa = sh + 2 * D, *sr = sh + 3 * D, *scratch = sh + 4 * D;
+  const int v = threadIdx.x;
+  const bool live = v < D;
+  const int entry = blockIdx.x, head = blockIdx.y;
+  const int row0 = p.q_start[entry], n_rows = p.q_start[entry + 1] - row0;
+  if (n_rows <= 0) return;
+  const int64_t col0 = (int64_t)head * D;
+  float* st = p.state + (int64_t)p.state_slots[entry] * p.state_stride + ((int64_t)head * D + (live ? v : 0)) * D;
+  if (live && p.positions[row0] == 0)
+    for (int c = 0; c < D; ++c) st[c] = 0.f;
+  for (int t = 0; t < n_rows; ++t) {
+    const int64_t row = row0 + t;
+    __syncthreads();
+    if (live) {
+      sk[v] = p.k[row * p.k_stride + col0 + v];
+      sw[v] = p.w_pre[row * p.w_stride + col0 + v];
+      sr[v] = p.r[row * p.r_stride + col0 + v];
+      sa[v] = RULE == RULE_DELTA ? p.a_pre[row * p.a_stride + col0 + v] : p.bonus[col0 + v];
+    }
+    const float kk = block_sum(live ? sk[v] * sk[v] : 0.f, scratch);   // (its barriers also publish the vectors)
+    if (!live) continue;
+    const float kn = 1.f / sqrtf(kk + 1e-6f);
+    const float vv = p.v[row * p.v_stride + col0 + v];
+    float o = 0.f;
+    if (RULE == RULE_DELTA) {
+      float us = 0.f;
+      for (int c = 0; c < D; ++c) us = fmaf(sk[c] * kn, st[c], us);
+      for (int c = 0; c < D; ++c) {
+        const float s = sw[c] * st[c] - (sa[c] * (sk[c] * kn)) * us + sk[c] * vv;
+        st[c] = s;
+        o = fmaf(s, sr[c], o);
+      }
+    } else {
+      for (int c = 0; c < D; ++c) {
+        const float kv = sk[c] * vv;
+        o = fmaf(st[c] + sa[c] * kv, sr[c], o);
+        st[c] = sw[c] * st[c] + kv;
+      }
+    }
+    p.o_raw[row * p.o_stride + col0 + v] = o;
+  }
+}
+
 // out = o / sqrt(mean_head(o^2) + eps) * norm_w * gate(g_pre), head by head: a wave a (row, head).
 template <typename T, int RULE>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, int64_t o_stride,
@@ -221,7 +271,10 @@ static int launch_scan(const ScanArgs& p, int entries, int rows, int dim, int ou
     SCAN_CASE(16, 16, 16) SCAN_CASE(24, 8, 16) SCAN_CASE(32, 16, 16) SCAN_CASE(40, 8, 16) SCAN_CASE(48, 16, 16)
     SCAN_CASE(56, 8, 16) SCAN_CASE(64, 16, 16) SCAN_CASE(80, 16, 8) SCAN_CASE(96, 16, 8) SCAN_CASE(112, 16, 8)
     SCAN_CASE(128, 16, 8)
-    default: return DLI_ERR_ARGUMENT;
+    default: {
+      const int threads = (dim + 63) / 64 * 64;
+      recurrent_scan_any_kernel<RULE><<<dim3(entries, p.heads), threads, (4 * dim + 16) * sizeof(float), stream>>>(p, dim);
+    }
   }
 #undef SCAN_CASE
   if (dli_launch_status() != DLI_OK) return DLI_ERR_LAUNCH;
@@ -234,11 +287,9 @@ static int launch_scan(const ScanArgs& p, int entries, int rows, int dim, int ou
   return dli_launch_status();
 }
 
-// Head sizes that the kernel is built for.
-extern "C" int dli_recurrent_scan_supports(int dim) {
-  if (dim < 16 || dim % 8 != 0 || dim > 128) return 0;
-  return dim <= 64 || dim % 16 == 0;
-}
+// Head sizes that are taken: 16 to 64 in steps of 8 and 80 to 128 in steps of 16 by the kernel
+// above, any other from 1 to 1024 by the slow one.
+extern "C" int dli_recurrent_scan_supports(int dim) { return dim >= 1 && dim <= 1024; }
 
 extern "C" int dli_recurrent_scan(const float* r, int64_t r_stride, const float* k, int64_t k_stride, const float* v,
                                   int64_t v_stride, const float* w_pre, int64_t w_stride, const float* a_pre,

@@ -1628,7 +1628,7 @@ def recurrent_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, w: torch.T
             _require(t.shape == (n, width), f"{name} must be [n, heads*dim]")
     _rows(out, "out", out.dtype)
     _require(out.shape[1] == width, "out must be [n, heads*dim]")
-    _require(recurrent_scan_supports(dim), f"the recurrence kernel takes heads of 16 to 128 in steps of 8 (16 above 64), not {dim}")
+    _require(recurrent_scan_supports(dim), f"the recurrence kernels take heads of 1 to 1024, not {dim}")
     _dense(norm_w, "norm_w", torch.float32, 1)
     _require(norm_w.shape[0] == width, "norm_w must hold heads*dim values")
     _require(state.is_cuda and state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1

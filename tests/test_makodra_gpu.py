@@ -256,7 +256,8 @@ def test_unit_queries_and_keys_value_mix_and_cache_write(ops):
 # ------------------------------------------------------------------------------ recurrences
 
 @pytest.mark.parametrize("rule", ["delta", "bonus"])
-@pytest.mark.parametrize("H,D", [(2, 16), (3, 24), (1, 48), (2, 64), (1, 80), (1, 128), (5, 40)])
+@pytest.mark.parametrize("H,D", [(2, 16), (3, 24), (1, 48), (2, 64), (1, 80), (1, 128), (5, 40), (2, 12), (1, 72), (1, 136),
+                                 (3, 1)])
 def test_recurrence_in_steps_against_whole(ops, rule, H, D):
     """Three requests of unequal length, run in steps that cut them anywhere (down to one row, and
     across the kernel's own batches of rows), in slots that are used again, against the plain rule
@@ -348,12 +349,25 @@ CONFIGS = {
     "attention": {"architecture": "Makodra", "vocab": 64, "width": 64, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
                   "layers": [attn(8, 2, 16, 32, 5, 0.3, True, 96), attn(8, 2, 16, 32, 64, 0.2, True, 96)]},
 }
+# shapes for the whole-prompt and mixed-batch tests only
+MORE_CONFIGS = {
+    # recurrent layers alone (no pages at all), heads whose size is no multiple of 16, an odd rank, an odd vocabulary
+    "recurrent_only": {"architecture": "Makodra", "vocab": 257, "width": 72, "norm": {"eps": 1e-5}, "logit_softcap": 9.0,
+                       "layers": [rec("wkv", 3, 24, 0, rank=5), rec("general_delta", 1, 40, 100), rec("general_delta", 2, 56, 0, rank=12),
+                                  rec("wkv", 1, 128, 88), rec("general_delta", 1, 96, 0)]},
+    # twelve query heads on one kv head, heads that the matrix-core kernel does not take, chunks of one and of
+    # more than any prompt, a page that is no multiple of eight keys
+    "wide_group": {"architecture": "Makodra", "vocab": 130, "width": 96, "norm": {"eps": 1e-6}, "logit_softcap": 50.0,
+                   "layers": [attn(12, 1, 24, 8, 1, 0.2, True, 0), attn(12, 1, 16, 8, 1000, 0.3, True, 64),
+                              attn(2, 2, 128, 96, 37, 0.05, False, 0), attn(12, 1, 40, 8, 9, 0.2, True, 0)]},
+}
+CONFIGS_ALL = {**CONFIGS, **MORE_CONFIGS}
 _MODELS: dict = {}
 
 
 def model(name: str, tmp_root):
     if name not in _MODELS:
-        cfg = CONFIGS[name]
+        cfg = CONFIGS_ALL[name]
         W = P.random_weights(cfg, seed=len(name) * 7 + 1)
         _MODELS[name] = (cfg, W, P.write_folder(tmp_root / name, cfg, W))
     return _MODELS[name]
@@ -425,7 +439,7 @@ def prompt(cfg, n, seed):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", list(CONFIGS))
+@pytest.mark.parametrize("name", list(CONFIGS_ALL))
 def test_whole_prompt_layers_and_logits(name, dtype, tmp_root):
     cfg, W, folder = model(name, tmp_root)
     toks = prompt(cfg, 70, 1)
@@ -473,15 +487,16 @@ def test_portions_of_every_size(name, dtype, tmp_root):
         close(torch.cat(rows), ref, dtype, (name, sizes))
 
 
+@pytest.mark.parametrize("page_size", [16, 4])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", list(CONFIGS))
-def test_mixed_batches_with_pages_and_slots_used_again(name, dtype, tmp_root):
+@pytest.mark.parametrize("name", list(CONFIGS_ALL))
+def test_mixed_batches_with_pages_and_slots_used_again(name, dtype, page_size, tmp_root):
     """Five unequal requests through two state slots and a pool that holds two of them at a time:
     portions of some beside single tokens of others; every request against itself alone."""
     cfg, W, folder = model(name, tmp_root)
     reqs = {i: prompt(cfg, n, 10 + i) for i, n in enumerate([90, 37, 1, 64, 55])}
     refs = {i: reference(W, cfg, t, dtype) for i, t in reqs.items()}
-    s = session(folder, dtype, pages=12, page_size=16, max_seqs=2, graphs=dtype == "bfloat16")
+    s = session(folder, dtype, pages=192 // page_size, page_size=page_size, max_seqs=2, graphs=dtype == "bfloat16")
     plan = [[(0, 30), (1, 5)], [(0, 1), (1, 30)], [(0, 2), (1, 1)], [(1, 1), (0, 40)], [(0, 1)], [(0, 16), (2, 1)],
             [(3, 33)], [(3, 1)], [(3, 30), (4, 2)], [(4, 1)], [(4, 1)], [(4, 50)], [(4, 1)]]
     at = {i: 0 for i in reqs}
