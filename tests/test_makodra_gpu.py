@@ -163,7 +163,7 @@ def test_attention_with_every_change_of_the_scores(ops, dtype, H, G, D, V, ps):
     kp, vp, table = paged(k, v, ps, dtype)
     tol = 1e-5 if dtype == torch.float32 else 3e-2
     cases = [dict(), dict(sink=True), dict(chunk=16), dict(chunk=7, sink=True), dict(window=9),
-             dict(r1=r1, r2=r2), dict(chunk=33, sink=True, r1=r1, r2=r2), dict(chunk=200, sink=True, r1=r1, r2=r2)]
+             dict(r1=r1, r2=r2), dict(chunk=33, sink=True, r1=r1, r2=r2), dict(chunk=300, sink=True, r1=r1, r2=r2)]
     for case in cases:
         pen = {n_: t.double() for n_, t in case.items() if n_ in ("r1", "r2")}
         ref = P.scored_attention_core(q, k, v, 0.7, chunk=case.get("chunk", 0), window=case.get("window", 0),
@@ -360,6 +360,10 @@ MORE_CONFIGS = {
     "wide_group": {"architecture": "Makodra", "vocab": 130, "width": 96, "norm": {"eps": 1e-6}, "logit_softcap": 50.0,
                    "layers": [attn(12, 1, 24, 8, 1, 0.2, True, 0), attn(12, 1, 16, 8, 1000, 0.3, True, 64),
                               attn(2, 2, 128, 96, 37, 0.05, False, 0), attn(12, 1, 40, 8, 9, 0.2, True, 0)]},
+    # nothing lines up: a width whose rows are not 16-byte aligned in bfloat16, heads of 20, 12 and 8, a rank of 3
+    "unaligned": {"architecture": "Makodra", "vocab": 77, "width": 100, "norm": {"eps": 1e-4}, "logit_softcap": 25.0,
+                  "layers": [attn(2, 1, 20, 12, 11, 0.2, True, 52), rec("general_delta", 5, 20, 0, rank=3), rec("wkv", 2, 8, 52, rank=3),
+                             attn(2, 1, 20, 12, 30, 0.2, True, 0)]},
 }
 CONFIGS_ALL = {**CONFIGS, **MORE_CONFIGS}
 _MODELS: dict = {}
