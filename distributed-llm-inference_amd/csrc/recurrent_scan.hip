@@ -37,7 +37,7 @@
 struct ScanArgs {
   const float* r; const float* k; const float* v;   // [rows][heads * D], each with its row stride
   const float* w_pre;                                // the decay w
-  const float* a_pre; const float* a_bias;           // RULE_DELTA: the removal rate a (a_bias is not read)
+  const float* a_pre; const float* a_bias;           // RULE_DELTA: the removal rate a (a_bias: unused, kept for the layout)
   const float* g_pre;                                // gate before its activation
   int64_t r_stride, k_stride, v_stride, w_stride, a_stride, g_stride;
   const float* bonus;                                // RULE_BONUS: [heads][D]
