@@ -9,7 +9,9 @@ Inside a page, keys lie as ``[kv_heads][page_size][head_dim]`` and values as
 ``[kv_heads][value_dim][page_size]`` (the order in which the attention kernels consume them).
 A mixer that declares a :class:`StateSpec` gets an array ``[state slots + 1, *shape]`` instead: one
 row per slot that a request can hold, and a last row (``scratch_slot``) that no request holds, for
-the padding rows of a replayed graph to write to.
+the padding rows of a replayed graph to write to. A mixer made of several such mixers declares a
+:class:`CompositeCacheSpec`; its cache holds one cache per member, each made as if the member were
+a layer of its own.
 Everything is allocated once and zero-filled (reference: src/dli/kv/paged_store.py:50-52).
 """
 
@@ -20,7 +22,7 @@ from typing import Optional, Sequence
 
 import torch
 
-from ..parts.base import PagedKVSpec, Runtime, StateSpec
+from ..parts.base import CompositeCacheSpec, PagedKVSpec, Runtime, StateSpec
 from .manager import CopyOp, GroupSpec
 
 
@@ -29,23 +31,41 @@ class LayerCache:
     """What one schedule entry's mixer gets: its pages (with the group whose block tables index
     them) or its state array. ``writable`` is False for an entry that reads another's cache."""
 
-    kind: str  # "paged" or "state"
+    kind: str  # "paged", "state" or "composite"
     group: int = -1
     k_pages: Optional[torch.Tensor] = None  # [pages, kv_heads, page_size, head_dim]
     v_pages: Optional[torch.Tensor] = None  # [pages, kv_heads, value_dim, page_size]; None: keys only
     state: Optional[torch.Tensor] = None    # [slots, *shape]
     writable: bool = True
     window: int = 0
+    members: Optional[dict] = None          # composite: member name -> LayerCache
 
     def reader(self) -> "LayerCache":
-        return LayerCache(self.kind, self.group, self.k_pages, self.v_pages, self.state, False, self.window)
+        members = None if self.members is None else {n: c.reader() for n, c in self.members.items()}
+        return LayerCache(self.kind, self.group, self.k_pages, self.v_pages, self.state, False, self.window, members)
+
+    def leaves(self) -> list["LayerCache"]:
+        """This cache, or the caches of a composite's members."""
+        return [self] if self.members is None else [leaf for c in self.members.values() for leaf in c.leaves()]
+
+
+def flatten_specs(specs: Sequence[Optional[PagedKVSpec | StateSpec | CompositeCacheSpec]]) -> list:
+    """Every paged or state spec in order, a composite's members in its place."""
+    flat: list = []
+    for s in specs:
+        if isinstance(s, CompositeCacheSpec):
+            flat.extend(m for _, m in s.members)
+        else:
+            flat.append(s)
+    return flat
 
 
 def plan_groups(specs: Sequence[Optional[PagedKVSpec | StateSpec]]) -> tuple[list[PagedKVSpec], list[int]]:
-    """Distinct paged specs in order of first appearance, and each layer's group (-1: none)."""
+    """Distinct paged specs in order of first appearance, and the group of each layer (or member
+    of a composite, counted as a layer in its place; -1: none)."""
     groups: list[PagedKVSpec] = []
     of_layer: list[int] = []
-    for s in specs:
+    for s in flatten_specs(specs):
         if isinstance(s, PagedKVSpec):
             if s not in groups:
                 groups.append(s)
@@ -86,27 +106,37 @@ class CacheStore:
             self.pools.append([torch.zeros(shape, device=rt.device, dtype=rt.dtype) for shape in shapes])
         self.layers: list[Optional[LayerCache]] = []
         seen = [0] * len(self.groups)
-        for spec, g in zip(specs, self._group_of):
+        at = 0   # index into the flattened list of specs, which is what the groups were planned from
+
+        def make(spec) -> Optional[LayerCache]:
+            nonlocal at
+            g = self._group_of[at]
+            at += 1
             if isinstance(spec, PagedKVSpec):
                 i = seen[g]
                 seen[g] += 1
                 pools = self.pools[g]
                 keys = pools[0][i, 0]
                 values = pools[0][i, 1] if pools[0].shape[1] == 2 else (pools[1][i, 0] if len(pools) > 1 else None)
-                self.layers.append(LayerCache(
+                return LayerCache(
                     "paged", g,
                     keys.view(num_pages, spec.kv_heads, page_size, spec.head_dim),
                     None if values is None else values.view(num_pages, spec.kv_heads, spec.v_dim, page_size),
-                    window=spec.window))
-            elif isinstance(spec, StateSpec):
-                self.layers.append(LayerCache(
-                    "state", state=torch.zeros(max_seqs + 1, *spec.shape, device=rt.device, dtype=spec.dtype)))
+                    window=spec.window)
+            if isinstance(spec, StateSpec):
+                return LayerCache(
+                    "state", state=torch.zeros(max_seqs + 1, *spec.shape, device=rt.device, dtype=spec.dtype))
+            return None
+
+        for spec in specs:
+            if isinstance(spec, CompositeCacheSpec):
+                self.layers.append(LayerCache("composite", members={name: make(m) for name, m in spec.members}))
             else:
-                self.layers.append(None)
+                self.layers.append(make(spec))
 
     @property
     def stateful(self) -> bool:
-        return any(c is not None and c.kind == "state" for c in self.layers)
+        return any(leaf.kind == "state" for c in self.layers if c is not None for leaf in c.leaves())
 
     def bytes_per_page(self) -> int:
         return bytes_per_page(self.groups, self.layers_per_group, self.page_size, self.rt.dtype)

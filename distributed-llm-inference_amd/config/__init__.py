@@ -3,6 +3,7 @@
 from .errors import ConfigError, MissingConfigKeyError, UnsupportedModelError
 from .llama import LlamaConfig, RopeConfig
 from .makodra import MakodraConfig, MakodraLayer
+from .miberax import MiberaxConfig, MiberaxLayer
 from .registry import (
     Architecture,
     load_config,
@@ -14,7 +15,7 @@ from .registry import (
 )
 
 __all__ = [
-    "Architecture", "ConfigError", "LlamaConfig", "MakodraConfig", "MakodraLayer", "MissingConfigKeyError", "RopeConfig",
+    "Architecture", "ConfigError", "LlamaConfig", "MakodraConfig", "MakodraLayer", "MiberaxConfig", "MiberaxLayer", "MissingConfigKeyError", "RopeConfig",
     "UnsupportedModelError", "load_config", "read_config_json", "register_architecture",
     "registered_architectures", "resolve_architecture", "unregister_architecture",
 ]

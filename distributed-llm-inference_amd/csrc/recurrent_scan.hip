@@ -316,3 +316,21 @@ extern "C" int dli_recurrent_scan(const float* r, int64_t r_stride, const float*
   return rule == RULE_DELTA ? launch_scan<RULE_DELTA>(p, entries, rows, dim, out_is_bf16, stream)
                             : launch_scan<RULE_BONUS>(p, entries, rows, dim, out_is_bf16, stream);
 }
+
+// The per-head norm and gate alone, for a recurrence whose own kernel leaves o in 32-bit:
+// out = o / sqrt(mean_head(o^2) + eps) * norm_w * gate(g_pre), gate_silu: silu, else sigmoid.
+// norm_w holds heads * dim values (a weight that the heads share is repeated by the caller).
+extern "C" int dli_head_norm_gate(const float* o, int64_t o_stride, const float* g_pre, int64_t g_stride,
+                                  const float* norm_w, float eps, void* out, int64_t out_stride, int rows, int heads,
+                                  int dim, int gate_silu, int out_is_bf16, hipStream_t stream) {
+  if (rows <= 0) return DLI_OK;
+  const int64_t width = (int64_t)heads * dim;
+  if (heads <= 0 || dim <= 0 || o_stride < width || g_stride < width || out_stride < width) return DLI_ERR_ARGUMENT;
+  const dim3 grid(rows, (heads + 3) / 4);
+  if (grid.y > 65535) return DLI_ERR_ARGUMENT;
+#define HNG(T, RULE) head_norm_gate_kernel<T, RULE><<<grid, 256, 0, stream>>>(o, o_stride, g_pre, g_stride, norm_w, eps, (T*)out, out_stride, heads, dim)
+  if (out_is_bf16) { if (gate_silu) HNG(bf16_t, RULE_BONUS); else HNG(bf16_t, RULE_DELTA); }
+  else { if (gate_silu) HNG(float, RULE_BONUS); else HNG(float, RULE_DELTA); }
+#undef HNG
+  return dli_launch_status();
+}

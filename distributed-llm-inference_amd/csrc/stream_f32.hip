@@ -14,6 +14,12 @@
 //                      receives the step's last row
 //   lowrank_out        y = bias + W2 act(t): the second half of a low-rank projection, 32-bit (W2 given transposed)
 //   qk_unit_cache      per-head unit RMS of q and k, value mixing, cache write
+//   rotary_cache       rotary rotation of q and k from 32-bit projections (pairs side by side or half a
+//                      head apart, the first rot_dims components of a head), cache write
+//   group_norm         out(T) = w * x / sqrt(mean_part(x^2) + eps), a row's equal consecutive parts each by
+//                      its own root mean square; with delta: x += delta first, in place
+//   branch_norm_mean   the mean of up to four branches' outputs, each first divided by its root mean
+//                      square over the row and multiplied by its own weight
 #include "common.h"
 
 template <typename T>
@@ -24,8 +30,11 @@ __global__ void embed_sinusoid_kernel(const T* __restrict__ table, const int* __
   const T* src = table + (int64_t)ids[row] * width;
   const float p = (float)positions[row];
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
-    const float angle = p * inv_freq[i >> 1];
-    const float sum = to_f32(src[i]) + ((i & 1) ? cosf(angle) : sinf(angle));
+    float sum = to_f32(src[i]);
+    if (inv_freq != nullptr) {   // (nullptr: the token's row alone)
+      const float angle = p * inv_freq[i >> 1];
+      sum += (i & 1) ? cosf(angle) : sinf(angle);
+    }
     out[row * width + i] = sum;
     if (rounded != nullptr) rounded[row * width + i] = (bf16_t)sum;
   }
@@ -198,6 +207,109 @@ __global__ void qk_unit_cache_kernel(const float* __restrict__ proj, int64_t str
   }
 }
 
+// cos and sin of position * freq with the product's rounding error taken back: the product's low
+// half (one fused multiply-add) turns the functions by their own derivatives.
+__device__ __forceinline__ void rotary_cos_sin(float position, float freq, float* c, float* s) {
+  const float hi = position * freq;
+  const float lo = fmaf(position, freq, -hi);
+  float sh, ch;
+  sincosf(hi, &sh, &ch);
+  *c = fmaf(-lo, sh, ch);
+  *s = fmaf(lo, ch, sh);
+}
+
+// proj [tokens][stride] float32 holds q (q_heads x dim), k (kv_heads x dim) and v (kv_heads x vdim) at
+// the given column offsets. The first rot_dims components of every q and k head are rotated by
+// position * inv_freq[i]: pair i is (2i, 2i+1) where `interleaved`, else (i, i + rot_dims/2); the
+// other components pass. q goes out in T; the rotated k and v go to the token's cache slot
+// (negative: not cached). A thread an element: it reads its partner from proj.
+template <typename T>
+__global__ void rotary_cache_kernel(const float* __restrict__ proj, int64_t stride, int q_off, int k_off, int v_off,
+                                    const int* __restrict__ positions, const float* __restrict__ inv_freq, int rot_dims,
+                                    int interleaved, T* __restrict__ q_out, const int* __restrict__ slots,
+                                    T* __restrict__ k_pages, T* __restrict__ v_pages, int q_heads, int kv_heads, int dim,
+                                    int vdim, int page_size) {
+  const int64_t row = blockIdx.x;
+  const float* pr = proj + row * stride;
+  const float p = (float)positions[row];
+  const int slot = slots[row];
+  const int64_t page = slot >= 0 ? slot / page_size : 0;
+  const int off = slot >= 0 ? slot % page_size : 0;
+  const int half = rot_dims / 2;
+  for (int i = threadIdx.x; i < (q_heads + kv_heads) * dim; i += blockDim.x) {
+    const int h = i / dim, c = i - h * dim;
+    const bool is_q = h < q_heads;
+    const float* src = is_q ? pr + q_off + (int64_t)h * dim : pr + k_off + (int64_t)(h - q_heads) * dim;
+    float y = src[c];
+    if (c < rot_dims) {
+      int pair, partner;
+      bool first;
+      if (interleaved) { pair = c >> 1; partner = c ^ 1; first = (c & 1) == 0; }
+      else { first = c < half; pair = first ? c : c - half; partner = first ? c + half : c - half; }
+      float cs, sn;
+      rotary_cos_sin(p, inv_freq[pair], &cs, &sn);
+      const float other = src[partner];
+      y = first ? y * cs - other * sn : y * cs + other * sn;
+    }
+    if (is_q) q_out[(row * q_heads + h) * dim + c] = from_f32<T>(y);
+    else if (slot >= 0) k_pages[((page * kv_heads + (h - q_heads)) * page_size + off) * dim + c] = from_f32<T>(y);
+  }
+  if (slot >= 0)
+    for (int i = threadIdx.x; i < kv_heads * vdim; i += blockDim.x) {
+      const int g = i / vdim, c = i - g * vdim;
+      v_pages[((page * kv_heads + g) * vdim + c) * page_size + off] = from_f32<T>(pr[v_off + i]);
+    }
+}
+
+// x [rows][width] float32 (with delta: x += delta first, stored); each of `groups` equal consecutive
+// parts of the row is divided by its own root mean square; out(T) = w * that.
+template <typename T>
+__global__ void group_norm_kernel(float* __restrict__ x, const float* __restrict__ delta, int64_t delta_stride,
+                                  const float* __restrict__ weight, T* __restrict__ out, int width, int groups, float eps) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  float* xr = x + row * width;
+  const int part = width / groups;
+  for (int g = 0; g < groups; ++g) {
+    float ss = 0.f;
+    for (int i = g * part + threadIdx.x; i < (g + 1) * part; i += blockDim.x) {
+      float f = xr[i];
+      if (delta != nullptr) {
+        f += delta[row * delta_stride + i];
+        xr[i] = f;
+      }
+      ss += f * f;
+    }
+    const float r = 1.f / sqrtf(block_sum(ss, scratch) / (float)part + eps);
+    // (each thread reads back what it wrote itself)
+    for (int i = g * part + threadIdx.x; i < (g + 1) * part; i += blockDim.x)
+      out[row * width + i] = from_f32<T>(weight[i] * (xr[i] * r));
+  }
+}
+
+struct BranchArgs {
+  const float* y[4]; int64_t stride[4]; const float* weight[4];
+  int count;
+};
+
+__global__ void branch_norm_mean_kernel(BranchArgs b, float* __restrict__ out, int width, float eps) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  float r[4];
+  for (int j = 0; j < b.count; ++j) {
+    const float* yr = b.y[j] + row * b.stride[j];
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) ss += yr[i] * yr[i];
+    r[j] = 1.f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+  }
+  const float share = 1.f / (float)b.count;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float sum = 0.f;
+    for (int j = 0; j < b.count; ++j) sum += b.weight[j][i] * (b.y[j][row * b.stride[j] + i] * r[j]);
+    out[row * width + i] = sum * share;
+  }
+}
+
 extern "C" {
 
 int dli_embed_sinusoid(const void* table, const int* ids, const int* positions, const float* inv_freq, float* out,
@@ -301,6 +413,52 @@ int dli_qk_unit_cache(const float* proj, int64_t stride, int q_off, int k_off, i
     qk_unit_cache_kernel<float><<<rows, 256, 0, stream>>>(proj, stride, q_off, k_off, v_off, (float*)q_out, lambda,
                                                           v_first_in, v_first_out, slots, (float*)k_pages,
                                                           (float*)v_pages, q_heads, kv_heads, dim, vdim, page_size, eps);
+  return dli_launch_status();
+}
+
+int dli_rotary_cache(const float* proj, int64_t stride, int q_off, int k_off, int v_off, const int* positions,
+                     const float* inv_freq, int rot_dims, int interleaved, void* q_out, const int* slots, void* k_pages,
+                     void* v_pages, int rows, int q_heads, int kv_heads, int dim, int vdim, int page_size, int is_bf16,
+                     hipStream_t stream) {
+  if (rows <= 0) return DLI_OK;
+  if (q_heads <= 0 || kv_heads <= 0 || dim <= 0 || vdim <= 0 || page_size <= 0 || rot_dims < 0 || rot_dims > dim ||
+      rot_dims % 2 || (rot_dims > 0 && inv_freq == nullptr))
+    return DLI_ERR_ARGUMENT;
+  if (is_bf16)
+    rotary_cache_kernel<bf16_t><<<rows, 256, 0, stream>>>(proj, stride, q_off, k_off, v_off, positions, inv_freq, rot_dims,
+                                                          interleaved, (bf16_t*)q_out, slots, (bf16_t*)k_pages,
+                                                          (bf16_t*)v_pages, q_heads, kv_heads, dim, vdim, page_size);
+  else
+    rotary_cache_kernel<float><<<rows, 256, 0, stream>>>(proj, stride, q_off, k_off, v_off, positions, inv_freq, rot_dims,
+                                                         interleaved, (float*)q_out, slots, (float*)k_pages,
+                                                         (float*)v_pages, q_heads, kv_heads, dim, vdim, page_size);
+  return dli_launch_status();
+}
+
+int dli_group_norm(float* x, const float* delta, int64_t delta_stride, const float* weight, void* out, int rows, int width,
+                   int groups, float eps, int is_bf16, hipStream_t stream) {
+  if (rows <= 0) return DLI_OK;
+  if (width <= 0 || groups <= 0 || width % groups || (delta != nullptr && delta_stride < width)) return DLI_ERR_ARGUMENT;
+  const int threads = width / groups >= 1024 ? 512 : 256;
+  if (is_bf16)
+    group_norm_kernel<bf16_t><<<rows, threads, 0, stream>>>(x, delta, delta_stride, weight, (bf16_t*)out, width, groups, eps);
+  else
+    group_norm_kernel<float><<<rows, threads, 0, stream>>>(x, delta, delta_stride, weight, (float*)out, width, groups, eps);
+  return dli_launch_status();
+}
+
+int dli_branch_norm_mean(const float* const* y, const int64_t* strides, const float* const* weights, int count, float* out,
+                         int rows, int width, float eps, hipStream_t stream) {
+  if (rows <= 0) return DLI_OK;
+  if (width <= 0 || count < 1 || count > 4) return DLI_ERR_ARGUMENT;
+  BranchArgs b;
+  b.count = count;
+  for (int j = 0; j < 4; ++j) {
+    const int s = j < count ? j : 0;
+    if (y[s] == nullptr || weights[s] == nullptr || strides[s] < width) return DLI_ERR_ARGUMENT;
+    b.y[j] = y[s]; b.stride[j] = strides[s]; b.weight[j] = weights[s];
+  }
+  branch_norm_mean_kernel<<<rows, 256, 0, stream>>>(b, out, width, eps);
   return dli_launch_status();
 }
 

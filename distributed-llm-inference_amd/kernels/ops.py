@@ -119,6 +119,25 @@ _SIGNATURES = {
     "dli_recurrent_scan": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr,
                            _c_i64, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr,
                            _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_rotary_cache": [_c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_group_norm": [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+    "dli_branch_norm_mean": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_float, _c_ptr],
+    "dli_head_norm_gate": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_float, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int,
+                           _c_int, _c_ptr],
+    "dli_gated_delta_max_taps": [],
+    "dli_conv_prepare": [_c_ptr, _c_i64, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr, _c_ptr,
+                         _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_gated_delta_scan": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_int,
+                             _c_int, _c_int, _c_int, _c_ptr],
+    "dli_poly_norm": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+    "dli_clamped_glu": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_float, _c_float, _c_int, _c_ptr],
+    "dli_router_choose": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr, _c_ptr, _c_ptr],
+    "dli_expert_tile_rows": [],
+    "dli_expert_products": [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                            _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_int, _c_ptr],
+    "dli_expert_combine": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int,
+                           _c_int, _c_int, _c_int, _c_ptr],
 }
 
 _lib: Optional[ctypes.CDLL] = None
@@ -1345,20 +1364,21 @@ def _rounded_copy(rounded: Optional[torch.Tensor], like: torch.Tensor) -> None:
         _require(rounded.shape == like.shape, "the rounded copy differs from the stream in shape")
 
 
-def embed_sinusoid(table: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor,
+def embed_sinusoid(table: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor, inv_freq: Optional[torch.Tensor],
                    out: torch.Tensor, rounded: Optional[torch.Tensor] = None) -> None:
     """``out[t] = table[ids[t]] + pe(positions[t])`` in float32, ``pe[2i] = sin(p f_i)``,
-    ``pe[2i+1] = cos(p f_i)`` with ``f = inv_freq [ceil(width/2)]``. ``rounded``: the same rows once
-    more in bfloat16."""
+    ``pe[2i+1] = cos(p f_i)`` with ``f = inv_freq [ceil(width/2)]`` (``None``: the token's row alone, widened
+    to float32). ``rounded``: the same rows once more in bfloat16."""
     _rounded_copy(rounded, out)
     _dense(table, "table", ndim=2)
     _dense(ids, "ids", torch.int32, 1)
     _dense(positions, "positions", torch.int32, 1)
-    _dense(inv_freq, "inv_freq", torch.float32, 1)
     _dense(out, "out", torch.float32, 2)
     n, width = ids.shape[0], table.shape[1]
     _require(positions.shape[0] == n and out.shape == (n, width), "ids, positions and out disagree on the rows")
-    _require(inv_freq.shape[0] * 2 >= width, "inv_freq must hold a frequency for every pair of columns")
+    if inv_freq is not None:
+        _dense(inv_freq, "inv_freq", torch.float32, 1)
+        _require(inv_freq.shape[0] * 2 >= width, "inv_freq must hold a frequency for every pair of columns")
     _check(library().dli_embed_sinusoid(_ptr(table), _ptr(ids), _ptr(positions), _ptr(inv_freq), _ptr(out), _ptr(rounded), n, width,
                                         _is_bf16(table.dtype), _stream()), "embed_sinusoid")
 
@@ -1650,3 +1670,265 @@ def recurrent_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, w: torch.T
         _ptr(a_bias), _ptr(g_pre), g_pre.stride(0), _ptr(bonus), _ptr(norm_w), float(eps), _ptr(state), state.stride(0),
         _ptr(q_start), _ptr(positions), _ptr(state_slots), _ptr(o_raw), o_raw.stride(0), _ptr(out), out.stride(0), entries,
         n, heads, dim, int(rule), _is_bf16(out.dtype), _stream()), "recurrent_scan")
+
+
+# ----------------------------------------------------------------------------- rotary keys from 32-bit projections
+
+def rotary_cache(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, positions: torch.Tensor,
+                 inv_freq: Optional[torch.Tensor], rot_dims: int, interleaved: bool, q_out: torch.Tensor,
+                 slots: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, q_heads: int) -> None:
+    """From the float32 projections ``proj [n, >= ...]`` (q at ``q_off``, k at ``k_off``, v at ``v_off``):
+    the first ``rot_dims`` components of every q and k head rotated by ``position * inv_freq[i]`` (pair
+    ``i`` is ``(2i, 2i+1)`` where ``interleaved``, else ``(i, i + rot_dims/2)``; 32-bit angles),
+    ``q_out [n, q_heads*dim]``; rotated k and v written at each token's cache slot."""
+    _f32_rows(proj, "proj")
+    _dense(k_pages, "k_pages", ndim=4)
+    dtype = k_pages.dtype
+    pages, kv_heads, page_size, dim = k_pages.shape
+    _dense(v_pages, "v_pages", dtype, 4)
+    vdim = v_pages.shape[2]
+    _require(v_pages.shape == (pages, kv_heads, vdim, page_size), "v_pages must be [pages, kv_heads, vdim, page_size]")
+    n = proj.shape[0]
+    _dense(q_out, "q_out", dtype, 2)
+    _require(q_out.shape == (n, q_heads * dim), "q_out must be [n, q_heads*dim]")
+    _dense(slots, "slots", torch.int32, 1)
+    _dense(positions, "positions", torch.int32, 1)
+    _require(slots.shape[0] == n and positions.shape[0] == n, "slots and positions differ from proj in rows")
+    for off, size in ((q_off, q_heads * dim), (k_off, kv_heads * dim), (v_off, kv_heads * vdim)):
+        _require(0 <= off and off + size <= proj.shape[1], "a projection lies outside proj's columns")
+    _require(0 <= rot_dims <= dim and rot_dims % 2 == 0, "the rotated components must be an even number within the head")
+    if rot_dims:
+        _dense(inv_freq, "inv_freq", torch.float32, 1)
+        _require(inv_freq.shape[0] * 2 == rot_dims, "inv_freq must hold rot_dims/2 frequencies")
+    _check(library().dli_rotary_cache(
+        _ptr(proj), proj.stride(0), q_off, k_off, v_off, _ptr(positions), _ptr(inv_freq if rot_dims else None), int(rot_dims),
+        int(bool(interleaved)), _ptr(q_out), _ptr(slots), _ptr(k_pages), _ptr(v_pages), n, q_heads, kv_heads, dim, vdim,
+        page_size, _is_bf16(dtype), _stream()), "rotary_cache")
+
+
+def group_norm(x: torch.Tensor, weight: torch.Tensor, groups: int, eps: float, out: torch.Tensor,
+               delta: Optional[torch.Tensor] = None) -> None:
+    """``out = weight * n(x)`` for a float32 ``x [rows, width]``, ``n`` dividing each of ``groups`` equal
+    consecutive parts of a row by its own root mean square (eps inside the root); 32-bit, rounded once
+    to ``out``'s type. With ``delta`` (float32, rows contiguous): ``x += delta`` first, in place."""
+    _dense(x, "x", torch.float32, 2)
+    _dense(weight, "weight", torch.float32, 1)
+    _dense(out, "out", ndim=2)
+    _require(out.shape == x.shape and weight.shape[0] == x.shape[1], "out, x and weight disagree on the sizes")
+    _require(groups >= 1 and x.shape[1] % groups == 0, "the row does not split into that many equal parts")
+    stride = 0
+    if delta is not None:
+        _f32_rows(delta, "delta")
+        _require(delta.shape == x.shape, "delta differs from x in shape")
+        stride = delta.stride(0)
+    _check(library().dli_group_norm(_ptr(x), _ptr(delta), stride, _ptr(weight), _ptr(out), x.shape[0], x.shape[1],
+                                    int(groups), float(eps), _is_bf16(out.dtype), _stream()), "group_norm")
+
+
+def branch_norm_mean(branches: Sequence[torch.Tensor], weights: Sequence[torch.Tensor], eps: float,
+                     out: torch.Tensor) -> None:
+    """``out = mean_j(weights[j] * branches[j] / sqrt(mean(branches[j]^2) + eps))`` row by row: up to four
+    float32 ``[rows, width]`` branches (rows contiguous), each normalised over the whole row."""
+    _dense(out, "out", torch.float32, 2)
+    count = len(branches)
+    _require(1 <= count <= 4 and len(weights) == count, "one to four branches, each with its weight")
+    for y, w in zip(branches, weights):
+        _f32_rows(y, "branch")
+        _dense(w, "weight", torch.float32, 1)
+        _require(y.shape == out.shape and w.shape[0] == out.shape[1], "a branch or its weight differs from out in size")
+    ys = (ctypes.c_void_p * count)(*[y.data_ptr() for y in branches])
+    strides = (ctypes.c_int64 * count)(*[y.stride(0) for y in branches])
+    ws = (ctypes.c_void_p * count)(*[w.data_ptr() for w in weights])
+    _check(library().dli_branch_norm_mean(ctypes.cast(ys, _c_ptr), ctypes.cast(strides, _c_ptr), ctypes.cast(ws, _c_ptr),
+                                          count, _ptr(out), out.shape[0], out.shape[1], float(eps), _stream()),
+           "branch_norm_mean")
+
+
+# ----------------------------------------------------------------------------- the gated delta rule
+
+def gated_delta_max_taps() -> int:
+    return int(library().dli_gated_delta_max_taps())
+
+
+def conv_prepare(proj: torch.Tensor, b_off: int, a_off: int, conv_w: torch.Tensor, a_log: torch.Tensor,
+                 dt_bias: torch.Tensor, state: torch.Tensor, kept_offset: int, q_start: torch.Tensor,
+                 positions: torch.Tensor, state_slots: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int,
+                 dim: int, vdim: int) -> None:
+    """What the gated delta rule reads, from a step's float32 projections ``proj [n, >=]`` (columns: q and
+    k, ``kv_heads x dim`` each, then v, ``heads x vdim``; beta's and the decay's pre-activations at ``b_off``
+    and ``a_off``): the short causal convolution per channel (``conv_w [channels, taps]``, the inputs before
+    the step's first row from ``state[slot, kept_offset:]``, which then receives the step's last
+    ``taps - 1`` inputs), silu, unit q and k per head (q times ``dim^-1/2``), ``beta = sigmoid(b)``,
+    ``g = exp(-exp(a_log) softplus(a + dt_bias))``; ``out [n, channels + 2 heads]`` float32."""
+    _f32_rows(proj, "proj")
+    _dense(conv_w, "conv_w", torch.float32, 2)
+    channels, taps = conv_w.shape
+    _require(channels == 2 * kv_heads * dim + heads * vdim, "conv_w must hold a row per channel of q, k and v")
+    _require(1 <= taps <= gated_delta_max_taps(), "too many taps")
+    for name, t in (("a_log", a_log), ("dt_bias", dt_bias)):
+        _dense(t, name, torch.float32, 1)
+        _require(t.shape[0] == heads, f"{name} must hold a value per head")
+    _dense(out, "out", torch.float32, 2)
+    n = proj.shape[0]
+    _require(out.shape == (n, channels + 2 * heads), "out must be [n, channels + 2 heads]")
+    _require(state.is_cuda and state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+             and state.shape[1] >= kept_offset + (taps - 1) * channels, "state must be float32 [slots, >= kept inputs]")
+    for name, t in (("q_start", q_start), ("positions", positions), ("state_slots", state_slots)):
+        _dense(t, name, torch.int32, 1)
+    entries = state_slots.shape[0]
+    _require(q_start.shape[0] == entries + 1 and positions.shape[0] == n, "q_start/state_slots/positions disagree")
+    _require(channels <= b_off and b_off + heads <= proj.shape[1] and channels <= a_off and a_off + heads <= proj.shape[1],
+             "beta's or the decay's columns lie outside proj")
+    _check(library().dli_conv_prepare(
+        _ptr(proj), proj.stride(0), int(b_off), int(a_off), _ptr(conv_w), _ptr(a_log), _ptr(dt_bias), _ptr(state),
+        state.stride(0), int(kept_offset), _ptr(q_start), _ptr(positions), _ptr(state_slots), _ptr(out), out.stride(0),
+        entries, n, heads, kv_heads, dim, vdim, taps, _stream()), "conv_prepare")
+
+
+def gated_delta_scan(prep: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor, positions: torch.Tensor,
+                     state_slots: torch.Tensor, o: torch.Tensor, heads: int, kv_heads: int, dim: int, vdim: int) -> None:
+    """Per request and head ``S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q`` over the step's rows
+    in order, ``S`` float32 ``[heads][vdim][dim]`` at the start of ``state[slot]`` (zeros at position 0);
+    ``prep`` as :func:`conv_prepare` leaves it; ``o [n, heads*vdim]`` float32."""
+    _f32_rows(prep, "prep")
+    _f32_rows(o, "o")
+    n = prep.shape[0]
+    _require(prep.shape[1] == 2 * kv_heads * dim + heads * vdim + 2 * heads, "prep must be [n, q | k | v | beta | g]")
+    _require(o.shape == (n, heads * vdim), "o must be [n, heads*vdim]")
+    _require(heads % kv_heads == 0, "heads do not group onto kv_heads")
+    _require(state.is_cuda and state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+             and state.shape[1] >= heads * vdim * dim, "state must be float32 [slots, >= heads*vdim*dim]")
+    for name, t in (("q_start", q_start), ("positions", positions), ("state_slots", state_slots)):
+        _dense(t, name, torch.int32, 1)
+    entries = state_slots.shape[0]
+    _require(q_start.shape[0] == entries + 1 and positions.shape[0] == n, "q_start/state_slots/positions disagree")
+    _check(library().dli_gated_delta_scan(
+        _ptr(prep), prep.stride(0), _ptr(state), state.stride(0), _ptr(q_start), _ptr(positions), _ptr(state_slots),
+        _ptr(o), o.stride(0), entries, n, heads, kv_heads, dim, vdim, _stream()), "gated_delta_scan")
+
+
+def head_norm_gate(o: torch.Tensor, g_pre: torch.Tensor, norm_w: torch.Tensor, eps: float, out: torch.Tensor,
+                   heads: int, dim: int, gate: str = "silu") -> None:
+    """``out = o / sqrt(mean_head(o^2) + eps) * norm_w * gate(g_pre)`` head by head: ``o`` and ``g_pre`` float32
+    ``[n, heads*dim]`` (rows contiguous), ``norm_w`` float32 ``[heads*dim]``, ``gate`` ``"silu"`` or ``"sigmoid"``."""
+    _f32_rows(o, "o")
+    _f32_rows(g_pre, "g_pre")
+    _rows(out, "out", out.dtype)
+    _dense(norm_w, "norm_w", torch.float32, 1)
+    n, width = o.shape[0], heads * dim
+    _require(o.shape == (n, width) and g_pre.shape == (n, width) and out.shape == (n, width) and norm_w.shape[0] == width,
+             "o, g_pre, out and norm_w must be [n, heads*dim]")
+    _require(gate in ("silu", "sigmoid"), "gate must be 'silu' or 'sigmoid'")
+    _check(library().dli_head_norm_gate(_ptr(o), o.stride(0), _ptr(g_pre), g_pre.stride(0), _ptr(norm_w), float(eps),
+                                        _ptr(out), out.stride(0), n, heads, dim, int(gate == "silu"),
+                                        _is_bf16(out.dtype), _stream()), "head_norm_gate")
+
+
+# ----------------------------------------------------------------------------- feed-forward: polynomial activation, experts
+
+def poly_norm(z: torch.Tensor, coef: torch.Tensor, eps: float, out: torch.Tensor) -> None:
+    """``out = a N(z) + b N(z^2) + c N(z^3) + e`` row by row, ``coef = (a, b, c, e)`` float32 on the device,
+    ``N(x) = x / sqrt(mean(x^2) + eps)``; ``z`` float32, ``out`` float32 or bfloat16."""
+    _f32_rows(z, "z")
+    _rows(out, "out", out.dtype)
+    _dense(coef, "coef", torch.float32, 1)
+    _require(coef.shape[0] == 4 and out.shape == z.shape, "four coefficients; out like z")
+    _check(library().dli_poly_norm(_ptr(z), z.stride(0), _ptr(coef), _ptr(out), out.stride(0), z.shape[0], z.shape[1],
+                                   float(eps), _is_bf16(out.dtype), _stream()), "poly_norm")
+
+
+def clamped_glu(gate_up: torch.Tensor, out: torch.Tensor, limit: float, alpha: float) -> None:
+    """``out = g sigmoid(alpha g) (u + 1)`` with ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)``;
+    ``gate_up [n, >= 2 ff]`` holds gate then up (rows contiguous), ``out [n, ff]`` of the same type."""
+    _rows(gate_up, "gate_up", out.dtype)
+    _dense(out, "out", ndim=2)
+    n, ff = out.shape
+    _require(gate_up.shape[0] == n and gate_up.shape[1] >= 2 * ff, "gate_up must hold gate and up for every row")
+    _check(library().dli_clamped_glu(_ptr(gate_up), gate_up.stride(0), _ptr(out), n, ff, float(limit), float(alpha),
+                                     _is_bf16(out.dtype), _stream()), "clamped_glu")
+
+
+def router_choose(logits: torch.Tensor, total: int, correction: Optional[torch.Tensor], groups: int, keep: int, top: int,
+                  scale: float, ids: torch.Tensor, weights: torch.Tensor) -> None:
+    """The router's choice per row of float32 ``logits [n, >= total]``: scores ``softmax`` over the first
+    ``total`` columns; choice scores add ``correction``; with ``groups`` > 1 only the ``keep`` groups of
+    neighbours with the largest best choice score can be chosen; ``ids [n, top]`` int32 are the largest
+    choice scores (lowest index on a tie), ``weights [n, top]`` their scores (without correction) divided
+    by their sum + 1e-20, times ``scale``."""
+    _f32_rows(logits, "logits")
+    n = logits.shape[0]
+    _require(logits.shape[1] >= total, "logits must hold every router output")
+    if correction is not None:
+        _dense(correction, "correction", torch.float32, 1)
+        _require(correction.shape[0] == total, "correction must hold a value per router output")
+    _dense(ids, "ids", torch.int32, 2)
+    _dense(weights, "weights", torch.float32, 2)
+    _require(ids.shape == (n, top) and weights.shape == (n, top), "ids and weights must be [n, top]")
+    _require(1 <= top <= min(total, 64) and groups >= 1 and total % groups == 0 and 1 <= keep <= groups
+             and keep * (total // groups) >= top, "the router's sizes do not fit each other")
+    _check(library().dli_router_choose(_ptr(logits), logits.stride(0), _ptr(correction), n, int(total), int(groups),
+                                       int(keep), int(top), float(scale), _ptr(ids), _ptr(weights), _stream()),
+           "router_choose")
+
+
+def expert_products(ids: torch.Tensor, h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
+                    limit: float, alpha: float) -> torch.Tensor:
+    """The chosen experts' results for every (token, choice): ``z [n * top, width]`` float32, row
+    ``t * top + j`` holding ``w_down[e] clamped_glu(w_gate[e] h_t, w_up[e] h_t)`` for ``e = ids[t, j]`` (rows of
+    ids at or above the number of experts are left unwritten). ``w_gate, w_up [experts, ff, width]``,
+    ``w_down [experts, width, ff]`` of ``h``'s type. Nothing here waits for the device: the rows are
+    sorted by expert and cut into tiles on the device."""
+    _dense(ids, "ids", torch.int32, 2)
+    n, top = ids.shape
+    _rows(h, "h", h.dtype)
+    for name, w in (("w_gate", w_gate), ("w_up", w_up), ("w_down", w_down)):
+        _dense(w, name, h.dtype, 3)
+    experts, ff, width = w_gate.shape
+    _require(w_up.shape == w_gate.shape and w_down.shape == (experts, width, ff) and h.shape == (n, width),
+             "h [n, width], w_gate/w_up [experts, ff, width], w_down [experts, width, ff] do not fit")
+    slots = n * top
+    tile_rows = int(library().dli_expert_tile_rows())
+    max_tiles = max(1, min(slots, slots // tile_rows + experts))
+    ints = torch.empty(experts + 1 + slots + 2 * max_tiles + 1, device=h.device, dtype=torch.int32)
+    offsets, order = ints[:experts + 1], ints[experts + 1:experts + 1 + slots]
+    tiles = ints[experts + 1 + slots:]
+    tile_expert, tile_row0, tile_count = tiles[:max_tiles], tiles[max_tiles:2 * max_tiles], tiles[2 * max_tiles:]
+    y = torch.empty(slots, ff, device=h.device, dtype=h.dtype)
+    z = torch.empty(slots, width, device=h.device, dtype=torch.float32)
+    _check(library().dli_expert_products(
+        _ptr(ids), _ptr(h), h.stride(0), _ptr(w_gate), _ptr(w_up), _ptr(w_down), _ptr(offsets), _ptr(order),
+        _ptr(tile_expert), _ptr(tile_row0), _ptr(tile_count), max_tiles, _ptr(y), _ptr(z), n, top, experts, width, ff,
+        float(limit), float(alpha), _is_bf16(h.dtype), _stream()), "expert_products")
+    return z
+
+
+def expert_combine(ids: torch.Tensor, weights: torch.Tensor, z: Optional[torch.Tensor], h: torch.Tensor, experts: int,
+                   out: torch.Tensor, shared: Optional[torch.Tensor] = None,
+                   shared_gate: Optional[torch.Tensor] = None) -> None:
+    """``out[t] = sum_j weights[t, j] * (z[t * top + j] if ids[t, j] < experts else h[t])
+    + sigmoid(shared_gate[t]) * shared[t]``; ``out`` float32 ``[n, width]``, ``shared`` float32 ``[n, width]``
+    and ``shared_gate`` float32 ``[n, 1]`` (a column of a wider matrix will do), both optional."""
+    _dense(ids, "ids", torch.int32, 2)
+    _dense(weights, "weights", torch.float32, 2)
+    n, top = ids.shape
+    _rows(h, "h", h.dtype)
+    _dense(out, "out", torch.float32, 2)
+    width = out.shape[1]
+    _require(weights.shape == (n, top) and h.shape == (n, width) and out.shape[0] == n, "ids, weights, h and out disagree")
+    if z is not None:
+        _dense(z, "z", torch.float32, 2)
+        _require(z.shape == (n * top, width), "z must be [n * top, width]")
+    else:
+        _require(experts == 0, "without z every chosen id must be an identity expert")
+    s_stride = g_stride = 0
+    if shared is not None:
+        _f32_rows(shared, "shared")
+        _require(shared.shape == (n, width), "shared must be [n, width]")
+        s_stride = shared.stride(0)
+    if shared_gate is not None:
+        _require(shared is not None and shared_gate.is_cuda and shared_gate.dtype == torch.float32
+                 and shared_gate.dim() == 2 and shared_gate.shape == (n, 1), "shared_gate must be float32 [n, 1] beside shared")
+        g_stride = shared_gate.stride(0)
+    _check(library().dli_expert_combine(_ptr(ids), _ptr(weights), _ptr(z), _ptr(h), h.stride(0), _ptr(shared_gate), g_stride,
+                                        _ptr(shared), s_stride, _ptr(out), n, top, int(experts), width, _is_bf16(h.dtype),
+                                        _stream()), "expert_combine")

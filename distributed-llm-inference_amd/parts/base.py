@@ -74,6 +74,22 @@ class StateSpec:
     dtype: torch.dtype = torch.float32
 
 
+@dataclass(frozen=True)
+class CompositeCacheSpec:
+    """A mixer made of several mixers that each keep something per request: ``members`` names every
+    member's own spec (pages or a state). The schedule entry's cache then is a composite too
+    (``LayerCache.members[name]``); paged members join the groups of equal specs like any layer's."""
+
+    members: tuple  # of (name, PagedKVSpec | StateSpec)
+
+    def __post_init__(self) -> None:
+        names = [n for n, _ in self.members]
+        if not names or len(set(names)) != len(names):
+            raise ValueError("a composite cache needs members with distinct names")
+        if any(not isinstance(s, (PagedKVSpec, StateSpec)) for _, s in self.members):
+            raise ValueError("a member of a composite cache keeps pages or a state")
+
+
 @dataclass
 class DecodeStream:
     """The residual stream of a step with few rows, in the form the fused decode kernels pass on:
@@ -229,7 +245,7 @@ class Mixer(Part):
     each request's rows in order and must not let one request's rows influence another's.
     """
 
-    def cache_spec(self) -> Optional[PagedKVSpec | StateSpec]:
+    def cache_spec(self) -> Optional[PagedKVSpec | StateSpec | CompositeCacheSpec]:
         return None
 
     def decode_plan(self, requests: int, max_keys: int) -> Hashable:

@@ -1,6 +1,8 @@
 """Pre-norm arrangement: ``x + mixer(norm(x))`` then ``x + feed_forward(norm(x))``
 (reference: src/dli/model/llama.py:194-213). The residual sums are made inside the norms that
-follow them (32-bit sum, rounded to the activation type, then normalised)."""
+follow them (32-bit sum, rounded to the activation type, then normalised). A layer may have no
+feed-forward; the stream may be 32-bit in a bfloat16 runtime (an embedding that hands out float32
+rows, parts that return their 32-bit sums), in which case nothing of it is ever rounded."""
 
 from __future__ import annotations
 
@@ -15,7 +17,7 @@ from .registry import register_part
 
 @register_part("block", "pre_norm")
 class PreNormBlock(Block):
-    roles = ("mixer_norm", "mixer", "feed_forward_norm", "feed_forward")
+    roles = ("mixer_norm", "mixer")   # and, unless the layer has no feed-forward, "feed_forward_norm" and "feed_forward"
 
     def __init__(self, runtime: Runtime) -> None:
         super().__init__(runtime)
@@ -27,6 +29,8 @@ class PreNormBlock(Block):
                 parts: Mapping[str, Part]) -> tuple[torch.Tensor, Optional[torch.Tensor]]:
         h = parts["mixer_norm"].forward(x, delta)          # x <- x + delta
         a = parts["mixer"].forward(h, ctx, cache)
+        if "feed_forward" not in parts:
+            return x, a
         h = parts["feed_forward_norm"].forward(x, a)       # x <- x + a
         f = parts["feed_forward"].forward(h, ctx)
         return x, f
@@ -41,7 +45,7 @@ class PreNormBlock(Block):
         step's launches. That loop hard-codes one order of work, so the answer is ``None`` unless
         this is exactly this class (a subclass must describe itself), each of the four parts
         names exactly the kind that the loop computes, and all agree on the width."""
-        if type(self) is not PreNormBlock:
+        if type(self) is not PreNormBlock or any(role not in parts for role in self.NATIVE_PARTS):
             return None
         fields = {role: parts[role].native_fields() for role in self.NATIVE_PARTS}
         if any(f is None or f.get("kind") != self.NATIVE_PARTS[role] for role, f in fields.items()):
@@ -53,6 +57,8 @@ class PreNormBlock(Block):
                 "eps2": n2["eps"]}
 
     def streams(self, ctx: Any, parts: Mapping[str, Part]) -> bool:
+        if "feed_forward" not in parts:
+            return False
         fused_norms = all(hasattr(parts[r], "fused_params") for r in ("mixer_norm", "feed_forward_norm"))
         return fused_norms and parts["mixer"].streams(ctx) and parts["feed_forward"].streams(ctx)
 

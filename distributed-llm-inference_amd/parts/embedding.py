@@ -15,31 +15,44 @@ from .spec import WeightSpec
 
 @register_part("embedding", "token_embedding")
 class TokenEmbedding(Embedding):
-    def __init__(self, runtime: Runtime, *, vocab_size: int, hidden_size: int) -> None:
+    def __init__(self, runtime: Runtime, *, vocab_size: int, hidden_size: int, weight_name: str = "weight",
+                 float32_rows: bool = False) -> None:
+        """``float32_rows``: the rows go out widened to float32 whatever the runtime's type, for a
+        model that keeps its residual stream in 32-bit (the table keeps the runtime's type)."""
         super().__init__(runtime)
         self.vocab_size, self.hidden_size = vocab_size, hidden_size
+        self.weight_name, self.float32_rows = weight_name, bool(float32_rows)
         self.weight: torch.Tensor | None = None
 
     def graph_capturable(self, page_size: int) -> bool:
         return True  # kernels on device arrays only
 
     def weight_specs(self) -> dict[str, WeightSpec]:
-        return {"weight": WeightSpec((self.vocab_size, self.hidden_size))}
+        return {self.weight_name: WeightSpec((self.vocab_size, self.hidden_size))}
 
     def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
-        self.weight = tensors["weight"]
+        self.weight = tensors[self.weight_name]
 
     def table(self) -> torch.Tensor:
         assert self.weight is not None
         return self.weight
 
     def forward(self, ids: torch.Tensor) -> torch.Tensor:
+        if self.float32_rows:
+            raise RuntimeError("this embedding hands its rows to the step: call forward_step(ctx)")
         out = self.rt.empty(ids.shape[0], self.hidden_size)
         ops.embedding(self.table(), ids, out)
         return out
 
+    def forward_step(self, ctx: Any) -> torch.Tensor:
+        if not self.float32_rows:
+            return self.forward(ctx.token_ids)
+        out = torch.empty(ctx.token_ids.shape[0], self.hidden_size, device=self.rt.device, dtype=torch.float32)
+        ops.embed_sinusoid(self.table(), ctx.token_ids, ctx.positions, None, out)
+        return out
+
     def streams(self, ctx) -> bool:
-        return self.rt.is_bf16
+        return self.rt.is_bf16 and not self.float32_rows  # the fused decode kernels keep a stream of the runtime's type
 
     def forward_stream(self, ids: torch.Tensor) -> DecodeStream:
         n = ids.shape[0]
@@ -59,15 +72,10 @@ class SinusoidalTokenEmbedding(TokenEmbedding):
 
     def __init__(self, runtime: Runtime, *, vocab_size: int, hidden_size: int, base: float = 10000.0,
                  weight_name: str = "weight") -> None:
-        super().__init__(runtime, vocab_size=vocab_size, hidden_size=hidden_size)
-        self.base, self.weight_name = float(base), weight_name
+        super().__init__(runtime, vocab_size=vocab_size, hidden_size=hidden_size, weight_name=weight_name,
+                         float32_rows=True)
+        self.base = float(base)
         self._inv_freq: Optional[torch.Tensor] = None
-
-    def weight_specs(self) -> dict[str, WeightSpec]:
-        return {self.weight_name: WeightSpec((self.vocab_size, self.hidden_size))}
-
-    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
-        self.weight = tensors[self.weight_name]
 
     def finalize(self) -> None:
         pairs = (self.hidden_size + 1) // 2

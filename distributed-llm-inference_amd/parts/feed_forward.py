@@ -126,3 +126,39 @@ class GatedMLP(FeedForward):
                         bias=self.b_gate_up, norm_w=norm_w, eps=eps, ssq_in=stream.ssq)
         stream.wrote(ops.skinny_gemm(act, self.w_down, w_tiled=self.w_down_tiled, epilogue=ops.SKINNY_RESIDUAL,
                                      stream=stream.x, bias=self.b_down))
+
+
+@register_part("feed_forward", "poly_norm_mlp")
+class PolyNormMLP(FeedForward):
+    """``down(act(up(x)))`` with the polynomial activation ``act(z) = a N(z) + b N(z^2) + c N(z^3) + e``:
+    powers element by element, ``N`` dividing a row of ``intermediate_size`` values by its root mean
+    square (eps inside the root), and the four numbers ``(a, b, c, e)`` one tensor of the checkpoint.
+    The first product leaves its 32-bit sums, the activation and its norms are 32-bit, and the result
+    is the second product's 32-bit sums (a residual stream's next summand)."""
+
+    def __init__(self, runtime: Runtime, *, hidden_size: int, intermediate_size: int, norm_eps: float = 1e-6,
+                 names: Optional[Mapping[str, str]] = None) -> None:
+        super().__init__(runtime)
+        self.hidden_size, self.intermediate_size, self.norm_eps = hidden_size, intermediate_size, float(norm_eps)
+        self.names = {"up": "up", "down": "down", "act": "act", **dict(names or {})}
+        self.w_up = self.w_down = self.coef = None
+
+    def graph_capturable(self, page_size: int) -> bool:
+        return True  # kernels on device arrays only
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        h, i = self.hidden_size, self.intermediate_size
+        return {self.names["up"]: WeightSpec((i, h)), self.names["down"]: WeightSpec((h, i)),
+                self.names["act"]: WeightSpec((4,), role="float32", init="norm")}
+
+    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        self.w_up, self.w_down = tensors[self.names["up"]], tensors[self.names["down"]]
+        self.coef = tensors[self.names["act"]].contiguous()
+
+    def forward(self, x: torch.Tensor, ctx: Any) -> torch.Tensor:
+        from .linear import linear_f32
+
+        z = linear_f32(self.rt, x, self.w_up)
+        act = self.rt.empty(x.shape[0], self.intermediate_size)
+        ops.poly_norm(z, self.coef, self.norm_eps, act)
+        return linear_f32(self.rt, act, self.w_down)

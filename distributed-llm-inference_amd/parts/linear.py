@@ -144,3 +144,13 @@ def linear_f32(rt: Runtime, x: torch.Tensor, weight: torch.Tensor, out: Optional
         ops.to_float(tmp, wide)
         out.copy_(wide)
     return out
+
+
+def stack_rows(matrices, multiple: int = 16) -> torch.Tensor:
+    """The matrices one below the other, filled up with zero rows to a multiple of ``multiple`` rows
+    (a product kernel's tiles then need no edge case)."""
+    stacked = torch.cat(list(matrices), dim=0)
+    pad = -stacked.shape[0] % multiple
+    if pad:
+        stacked = torch.cat([stacked, stacked.new_zeros(pad, stacked.shape[1])], dim=0)
+    return stacked.contiguous()

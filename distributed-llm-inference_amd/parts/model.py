@@ -20,7 +20,9 @@ from .registry import build_part
 from .spec import ModelSpec, WeightSpec
 
 # importing the modules registers the built-in parts
-from . import attention, block, embedding, feed_forward, head, norm, position, recurrent, scored_attention  # noqa: F401,E402
+from . import (  # noqa: F401,E402
+    attention, block, embedding, experts, feed_forward, head, norm, parallel, position, recurrent, scored_attention,
+)
 
 
 @dataclass

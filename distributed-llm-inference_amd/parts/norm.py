@@ -67,3 +67,35 @@ class RMSNorm(Norm):
         else:
             ops.rms_norm(x, self.weight, self.eps, out, delta=delta, sum_out=x)
         return out
+
+
+@register_part("norm", "group_rms_norm")
+class GroupRMSNorm(Norm):
+    """RMS norm in groups, on a 32-bit residual stream: a row is split into ``groups`` equal
+    consecutive parts, each is divided by its own ``sqrt(mean(part^2) + eps)``, and the whole is
+    multiplied by the weight. Statistics and products are 32-bit; the result is rounded once, to the
+    type that the product after the norm reads. ``groups=1`` is the plain RMS norm of such a stream.
+    It offers no ``fused_params``: the kernels that compute a norm inside a product compute the plain one."""
+
+    def __init__(self, runtime: Runtime, *, width: int, eps: float, groups: int = 1, weight_name: str = "weight") -> None:
+        super().__init__(runtime)
+        if groups < 1 or width % groups:
+            raise ValueError(f"a row of {width} does not split into {groups} equal parts")
+        self.width, self.eps, self.groups, self.weight_name = width, float(eps), int(groups), weight_name
+        self.weight: torch.Tensor | None = None
+
+    def graph_capturable(self, page_size: int) -> bool:
+        return True  # kernels on device arrays only
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        return {self.weight_name: WeightSpec((self.width,), role="float32", init="norm")}
+
+    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        self.weight = tensors[self.weight_name]
+
+    def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if x.dtype != torch.float32:
+            raise RuntimeError("group_rms_norm normalises a float32 residual stream")
+        out = self.rt.empty(*x.shape)
+        ops.group_norm(x, self.weight, self.groups, self.eps, out, delta=delta)
+        return out

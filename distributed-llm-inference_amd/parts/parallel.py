@@ -1,0 +1,69 @@
+"""Mixers side by side: every branch reads the same rows, each branch's output is divided by its
+root mean square over the model width and multiplied by a weight of its own (a plain weight, not
+one plus it), and the result is the mean of the branches.
+
+The branches are mixers of any kind, given as part specs with their own tensor prefixes; each keeps
+whatever it keeps per request (pages, a state, nothing), and the pair's cache is the composite of
+theirs. Norms, weights and the mean are 32-bit, and so is the result (it is a residual stream's
+next summand)."""
+
+from __future__ import annotations
+
+from typing import Any, Mapping, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import CompositeCacheSpec, Mixer, Runtime
+from .registry import build_part, register_part
+from .spec import PartSpec, WeightSpec
+
+
+@register_part("mixer", "parallel_mixers")
+class ParallelMixers(Mixer):
+    MAX_BRANCHES = 4  # what the kernel that normalises and averages takes
+
+    def __init__(self, runtime: Runtime, *, hidden_size: int, branches: Mapping[str, PartSpec], norm_eps: float = 1e-6,
+                 out_weight_names: Optional[Mapping[str, str]] = None) -> None:
+        """``branches``: name -> the branch's mixer. ``out_weight_names``: name -> the tensor (below
+        this part's prefix) that multiplies the branch's normalised output; default ``<name>.out``."""
+        super().__init__(runtime)
+        if not 1 <= len(branches) <= self.MAX_BRANCHES:
+            raise ValueError(f"one to {self.MAX_BRANCHES} branches, not {len(branches)}")
+        self.hidden_size, self.norm_eps = hidden_size, float(norm_eps)
+        self.names = list(branches)
+        self.branches = {name: build_part("mixer", spec, runtime) for name, spec in branches.items()}
+        self.out_names = {name: (out_weight_names or {}).get(name, f"{name}.out") for name in self.names}
+        self.out_w: dict[str, torch.Tensor] = {}
+
+    def sub_parts(self) -> dict:
+        return dict(self.branches)
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        return {self.out_names[n]: WeightSpec((self.hidden_size,), role="float32", init="norm") for n in self.names}
+
+    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        self.out_w = {n: tensors[self.out_names[n]].contiguous() for n in self.names if self.out_names[n] in tensors}
+
+    def cache_spec(self) -> Optional[Any]:
+        members = tuple((n, b.cache_spec()) for n, b in self.branches.items() if b.cache_spec() is not None)
+        if not members:
+            return None
+        return CompositeCacheSpec(members)
+
+    def graph_capturable(self, page_size: int) -> bool:
+        return all(b.graph_capturable(page_size) for b in self.branches.values())
+
+    def forward(self, x: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:
+        members = cache.members if cache is not None and cache.kind == "composite" else {}
+        outs = []
+        for name in self.names:
+            y = self.branches[name].forward(x, ctx, members.get(name))
+            if y.dtype != torch.float32:
+                wide = torch.empty(y.shape, device=y.device, dtype=torch.float32)
+                ops.to_float(y, wide)
+                y = wide
+            outs.append(y)
+        out = torch.empty(x.shape[0], self.hidden_size, device=self.rt.device, dtype=torch.float32)
+        ops.branch_norm_mean(outs, [self.out_w[n] for n in self.names], self.norm_eps, out)
+        return out

@@ -52,9 +52,13 @@ _TABLES: dict = {}
 class Rotary(PositionEncoding):
     def __init__(self, runtime: Runtime, *, dim: int, theta: float, rope_type: str = "default",
                  factor: float = 1.0, low_freq_factor: float = 1.0, high_freq_factor: float = 4.0,
-                 original_max_position_embeddings: int = 8192) -> None:
+                 original_max_position_embeddings: int = 8192, pairing: str = "half") -> None:
+        """``pairing``: which components turn together: ``"half"`` (``i`` with ``i + dim/2``) or
+        ``"interleaved"`` (``2i`` with ``2i + 1``). The mixer's kernels must implement it."""
         super().__init__(runtime)
-        self.dim = dim
+        if pairing not in ("half", "interleaved"):
+            raise ValueError(f"unknown rotary pairing {pairing!r}")
+        self.dim, self.pairing = dim, pairing
         self.inv_freq_host = rotary_inverse_frequencies(
             dim, theta, rope_type, factor, low_freq_factor, high_freq_factor,
             original_max_position_embeddings)
@@ -75,7 +79,7 @@ class Rotary(PositionEncoding):
     def rotary_table(self) -> Optional[RotaryTable]:
         if self._table is None:
             self.finalize()
-        return RotaryTable(self._table, self.dim, "half")
+        return RotaryTable(self._table, self.dim, self.pairing)
 
 
 @register_part("position", "none")

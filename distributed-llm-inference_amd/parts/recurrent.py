@@ -1,6 +1,7 @@
 """Mixers that carry a matrix state per head from token to token instead of a cache of keys:
-``general_delta`` (a generalized delta rule) and ``wkv`` (decayed sums with a bonus for the current
-token and token shift). The state lives in 32-bit in the request's state slot
+``general_delta`` (a generalized delta rule), ``wkv`` (decayed sums with a bonus for the current
+token and token shift) and ``gated_delta`` (the delta rule with one decay and one write strength per
+head, behind short convolutions). The state lives in 32-bit in the request's state slot
 (:class:`StateSpec`), starts at zero at position 0, and is all that a step leaves for the next.
 
 Both run their projections as products of the runtime's type with 32-bit sums, and everything
@@ -17,7 +18,7 @@ import torch
 
 from ..kernels import ops
 from .base import Mixer, Runtime, StateSpec
-from .linear import as_operand, linear_f32
+from .linear import as_operand, linear_f32, stack_rows
 from .registry import register_part
 from .spec import WeightSpec
 
@@ -156,4 +157,77 @@ class WKV(_MatrixStateMixer):
         out = self.rt.empty(n, c)
         ops.recurrent_scan(r, k, v, w, g, self.norm_w, self.norm_eps, state[:, h:], ctx.q_start, ctx.positions,
                            ctx.state_slots, out, self.num_heads, self.head_dim, self.rule, bonus=self.bonus)
+        return linear_f32(self.rt, out, self.w_o)
+
+
+@register_part("mixer", "gated_delta")
+class GatedDelta(Mixer):
+    """The gated delta rule. From the rows ``h``: q and k (``num_kv_heads x head_dim``) and v (``num_heads x
+    value_dim``) each pass a short causal convolution over time per channel (``conv_taps`` taps, zeros
+    before position 0) and silu; q and k become unit vectors per head, ``x / sqrt(sum x^2 + 1e-6)``, q also
+    times ``head_dim^-1/2``; value head ``i`` reads q/k head ``i // (num_heads / num_kv_heads)``;
+    ``beta = sigmoid(W_b h)`` and ``g = exp(-exp(A_log) softplus(W_a h + dt_bias))`` per head. Per head
+    ``S <- g S``, ``u = beta (v - S^T k)``, ``S <- S + k u^T``, ``o = S^T q``; then
+    ``o / rms(o) * norm * silu(W_g h)`` (``norm`` of ``value_dim`` values, shared by the heads) and the
+    output product. The request's state slot holds ``S`` and the last ``conv_taps - 1`` inputs of the
+    convolutions, all 32-bit; everything between the projections and the output product is 32-bit."""
+
+    def __init__(self, runtime: Runtime, *, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 value_dim: int, conv_taps: int = 4, norm_eps: float = 1e-6) -> None:
+        super().__init__(runtime)
+        if num_heads < 1 or num_kv_heads < 1 or num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} heads do not group onto {num_kv_heads} q/k heads")
+        if head_dim < 1 or value_dim < 1 or not 1 <= conv_taps <= 16:
+            raise ValueError("head sizes must be positive and the convolution have 1 to 16 taps")
+        self.hidden_size, self.num_heads, self.num_kv_heads = hidden_size, num_heads, num_kv_heads
+        self.head_dim, self.value_dim, self.conv_taps, self.norm_eps = head_dim, value_dim, conv_taps, float(norm_eps)
+        self.qk, self.hv = num_kv_heads * head_dim, num_heads * value_dim
+        self.channels = 2 * self.qk + self.hv
+        self.state_floats = num_heads * value_dim * head_dim
+        self.w_in = self.conv_w = self.a_log = self.dt_bias = self.norm_w = self.w_o = None
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        h, t = self.hidden_size, self.conv_taps
+        return {"q": WeightSpec((self.qk, h)), "k": WeightSpec((self.qk, h)), "v": WeightSpec((self.hv, h)),
+                "q.conv": WeightSpec((self.qk, t), role="float32"),
+                "k.conv": WeightSpec((self.qk, t), role="float32"),
+                "v.conv": WeightSpec((self.hv, t), role="float32"),
+                "b": WeightSpec((self.num_heads, h)), "a": WeightSpec((self.num_heads, h)),
+                "A_log": WeightSpec((self.num_heads,), role="float32", init="zeros"),
+                "dt_bias": WeightSpec((self.num_heads,), role="float32", init="zeros"),
+                "norm": WeightSpec((self.value_dim,), role="float32", init="norm"),
+                "g": WeightSpec((self.hv, h)), "o": WeightSpec((h, self.hv))}
+
+    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        # one product for everything that reads h: q, k, v (the convolutions' channels, in this order),
+        # the gate, beta and the decay
+        self.w_in = stack_rows([tensors[n] for n in ("q", "k", "v", "g", "b", "a")])
+        self.conv_w = torch.cat([tensors[n] for n in ("q.conv", "k.conv", "v.conv")], dim=0).contiguous()
+        self.a_log, self.dt_bias = tensors["A_log"].contiguous(), tensors["dt_bias"].contiguous()
+        self.norm_w = tensors["norm"].repeat(self.num_heads).contiguous()   # the kernel reads a value per head and column
+        self.w_o = tensors["o"]
+
+    def cache_spec(self) -> StateSpec:
+        return StateSpec((self.state_floats + (self.conv_taps - 1) * self.channels,), torch.float32)
+
+    def graph_capturable(self, page_size: int) -> bool:
+        return True  # kernels on the context's device arrays only; padding rows write the spare slot
+
+    def forward(self, x: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:
+        if cache is None or cache.kind != "state" or not cache.writable:
+            raise RuntimeError("gated_delta needs a state of its own")
+        state = cache.state.view(cache.state.shape[0], -1)
+        n, H = x.shape[0], self.num_heads
+        proj = linear_f32(self.rt, as_operand(self.rt, x, ctx), self.w_in)
+        g_off = self.channels
+        b_off, a_off = g_off + self.hv, g_off + self.hv + H
+        prep = torch.empty(n, self.channels + 2 * H, device=self.rt.device, dtype=torch.float32)
+        ops.conv_prepare(proj, b_off, a_off, self.conv_w, self.a_log, self.dt_bias, state, self.state_floats,
+                         ctx.q_start, ctx.positions, ctx.state_slots, prep, H, self.num_kv_heads, self.head_dim,
+                         self.value_dim)
+        o = torch.empty(n, self.hv, device=self.rt.device, dtype=torch.float32)
+        ops.gated_delta_scan(prep, state, ctx.q_start, ctx.positions, ctx.state_slots, o, H, self.num_kv_heads,
+                             self.head_dim, self.value_dim)
+        out = self.rt.empty(n, self.hv)
+        ops.head_norm_gate(o, proj[:, g_off:g_off + self.hv], self.norm_w, self.norm_eps, out, H, self.value_dim, gate="silu")
         return linear_f32(self.rt, out, self.w_o)

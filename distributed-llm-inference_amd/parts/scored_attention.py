@@ -1,7 +1,7 @@
 """Grouped-query attention over the paged cache whose scores are changed by parameters: unit-RMS
-queries and keys, a per-head logarithmic distance penalty, a chunked mask, a softmax with a sink,
-value mixing across layers, and a sigmoid output gate. Each is a parameter that is off by default,
-so another design may take any subset.
+queries and keys or a rotary position encoding, a per-head logarithmic distance penalty, a chunked
+mask, a softmax with a sink, value mixing across layers, and a sigmoid output gate. Each is a
+parameter, so another design may take any subset.
 
 Order of work for the rows ``h`` of a step (``x`` may be a 32-bit residual stream; the products read
 it in the runtime's type):
@@ -11,6 +11,9 @@ it in the runtime's type):
 2. one kernel divides every head's q and k by its root mean square over ``dim`` (``qk_unit``), mixes
    v with the values that the first such layer of the step computed for the same token
    (``value_mix``: ``v <- (1 - m) v + m v_first``), and writes k and the mixed v into the cache pages;
+   with ``qk_unit=False`` the kernel instead rotates q and k as the ``position`` part's rotary table
+   says (any leading part of a head, pairs side by side or half a head apart; no table: q and k as
+   projected) and writes k and v into the pages;
 3. the attention kernel: ``s_ij = scale (q_i . k_j) - r1_h log(1 + r2_h (i - j))`` for ``j <= i`` in
    the same chunk of ``chunk`` positions (counted from the request's position 0), weights
    ``exp(s_ij) / (sink + sum_j exp(s_ij))`` with ``sink = 1`` (a key of score 0 that has no value),
@@ -28,10 +31,10 @@ from typing import Any, Mapping, Optional
 import torch
 
 from ..kernels import ops
-from .base import Mixer, PagedKVSpec, Runtime
+from .base import Mixer, PagedKVSpec, PositionEncoding, Runtime
 from .linear import as_operand, linear_f32
-from .registry import register_part
-from .spec import WeightSpec
+from .registry import build_part, register_part
+from .spec import PartSpec, WeightSpec
 
 
 @register_part("mixer", "scored_attention")
@@ -42,7 +45,8 @@ class ScoredAttention(Mixer):
                  value_dim: Optional[int] = None, scale: Optional[float] = None, qk_unit: bool = True,
                  norm_eps: float = 1e-6, distance_penalty: bool = False, chunk: int = 0, window: int = 0,
                  sink: bool = False, output_gate: bool = False, value_mix: str = "none",
-                 value_mix_key: str = "first_values", names: Optional[Mapping[str, str]] = None) -> None:
+                 value_mix_key: str = "first_values", names: Optional[Mapping[str, str]] = None,
+                 position: Optional[PartSpec] = None) -> None:
         super().__init__(runtime)
         if num_heads < 1 or num_kv_heads < 1 or num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads do not group onto {num_kv_heads} kv heads")
@@ -60,8 +64,11 @@ class ScoredAttention(Mixer):
         self.distance_penalty, self.chunk, self.window = bool(distance_penalty), int(chunk), int(window)
         self.sink, self.output_gate = bool(sink), bool(output_gate)
         self.value_mix, self.value_mix_key = value_mix, value_mix_key
-        if not self.qk_unit:
-            raise ValueError("scored_attention caches unit keys: qk_unit=False has no kernel")
+        self.position = build_part("position", position or PartSpec("none"), runtime)
+        if self.qk_unit and position is not None and position.kind != "none":
+            raise ValueError("scored_attention: unit keys and a position encoding together have no kernel")
+        if not self.qk_unit and value_mix != "none":
+            raise ValueError("scored_attention: value mixing belongs to the kernel that makes unit keys")
         self.names = {"q": "q", "k": "k", "v": "v", "g": "g", "o": "o", "mix": "vmix", "r1": "r1", "r2": "r2",
                       **dict(names or {})}
         self.w_in = self.w_o = self.mix = self.r1 = self.r2 = None
@@ -107,6 +114,17 @@ class ScoredAttention(Mixer):
         if self.value_mix == "mix":
             self.mix = tensors[n["mix"]].reshape(1).contiguous()
 
+    def sub_parts(self) -> dict:
+        return {"position": self.position}
+
+    def finalize(self) -> None:
+        table = self.position.rotary_table()
+        if table is not None and (table.dim > self.head_dim or table.pairing not in ("half", "interleaved")):
+            raise ops.KernelArgumentError(f"scored_attention cannot rotate {table.dim} of {self.head_dim} components "
+                                          f"with the pairing {table.pairing!r}")
+        if table is None and type(self.position).apply is not PositionEncoding.apply:
+            raise ops.KernelArgumentError("scored_attention takes a rotary table or no position encoding")
+
     def cache_spec(self) -> PagedKVSpec:
         return PagedKVSpec(self.num_kv_heads, self.head_dim, self.window,
                            None if self.value_dim == self.head_dim else self.value_dim)
@@ -129,9 +147,15 @@ class ScoredAttention(Mixer):
             first_in = ctx._memo.get(("value mix", self.value_mix_key))
             if first_in is None or first_in.shape != (n, self._v):
                 raise RuntimeError("value mixing needs an earlier layer of the step that keeps its values, of the same size")
-        ops.qk_unit_cache(proj, 0, self._q, self._q + self._k, q, grp.slots, cache.k_pages, cache.v_pages,
-                          self.num_heads, self.norm_eps, mix=self.mix if self.value_mix == "mix" else None,
-                          v_first_in=first_in, v_first_out=first_out)
+        if self.qk_unit:
+            ops.qk_unit_cache(proj, 0, self._q, self._q + self._k, q, grp.slots, cache.k_pages, cache.v_pages,
+                              self.num_heads, self.norm_eps, mix=self.mix if self.value_mix == "mix" else None,
+                              v_first_in=first_in, v_first_out=first_out)
+        else:
+            table = self.position.rotary_table()
+            ops.rotary_cache(proj, 0, self._q, self._q + self._k, ctx.positions, None if table is None else table.inv_freq,
+                             0 if table is None else table.dim, table is not None and table.pairing == "interleaved",
+                             q, grp.slots, cache.k_pages, cache.v_pages, self.num_heads)
         out = self.rt.empty(n, self._o)
         gate = proj[:, self._q + self._k + self._v:] if self.output_gate else None
         changes = dict(window=self.window, chunk=self.chunk, sink=self.sink, r1=self.r1, r2=self.r2)
