@@ -62,7 +62,7 @@ class RoutedExperts(FeedForward):
         h, f = self.hidden_size, self.expert_size
         specs = {"router": WeightSpec((self.total, h))}
         if self.has_correction:
-            specs["correction"] = WeightSpec((self.total,), role="float32", init="zeros")
+            specs["correction"] = WeightSpec((self.total,), role="float32", init="zeros", optional=True)
         for e in range(self.experts):
             specs.update({f"e{e}.gate": WeightSpec((f, h)), f"e{e}.up": WeightSpec((f, h)), f"e{e}.down": WeightSpec((h, f))})
         if self.shared_size:
@@ -75,7 +75,8 @@ class RoutedExperts(FeedForward):
     def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
         rows = [tensors["router"]] + ([tensors["shared.sg"]] if self.shared_gate else [])
         self.w_router = stack_rows(rows)
-        self.correction = tensors["correction"].contiguous() if self.has_correction else None
+        # (a checkpoint without the tensor: scores are chosen as they are)
+        self.correction = tensors["correction"].contiguous() if self.has_correction and "correction" in tensors else None
         if self.experts:
             self.w_gate = torch.stack([tensors[f"e{e}.gate"] for e in range(self.experts)]).contiguous()
             self.w_up = torch.stack([tensors[f"e{e}.up"] for e in range(self.experts)]).contiguous()

@@ -204,3 +204,112 @@ def forward(cfg: dict, tensors: dict, tokens, return_layers: bool = False):
         streams.append(x)
     logits = group_norm(x, t["final.norm"], groups, eps) @ t["embed"].T
     return (logits, torch.stack(streams)) if return_layers else logits
+
+
+forward_logits = forward
+
+
+def greedy_generate(cfg: dict, tensors: dict, prompt, n_new: int) -> list[int]:
+    toks, out = list(prompt), []
+    for _ in range(n_new):
+        nxt = int(forward(cfg, tensors, toks)[-1].argmax())
+        out.append(nxt)
+        toks.append(nxt)
+    return out
+
+
+# ------------------------------------------------------------------------------ weights of a test model
+
+def tensor_shapes(cfg: dict) -> dict[str, tuple]:
+    """Name -> shape of every tensor of a model of this configuration."""
+    w = cfg["width"]
+    out = {"embed": (cfg["vocab"], w), "final.norm": (w,)}
+    for i, layer in enumerate(cfg["layers"]):
+        out[f"l{i}.norm1"] = (w,)
+        a, d = layer["mixer"]["left"], layer["mixer"]["right"]
+        p = f"l{i}.mix.left."
+        out.update({p + "q": (a["heads"] * a["dim"], w), p + "k": (a["kv_heads"] * a["dim"], w),
+                    p + "v": (a["kv_heads"] * a["vdim"], w), p + "o": (w, a["heads"] * a["vdim"]), p + "out": (w,)})
+        p = f"l{i}.mix.right."
+        qk, hv, taps = d["kv_heads"] * d["dim"], d["heads"] * d["vdim"], d["conv"]
+        out.update({p + "q": (qk, w), p + "k": (qk, w), p + "v": (hv, w), p + "q.conv": (qk, taps), p + "k.conv": (qk, taps),
+                    p + "v.conv": (hv, taps), p + "b": (d["heads"], w), p + "a": (d["heads"], w), p + "A_log": (d["heads"],),
+                    p + "dt_bias": (d["heads"],), p + "norm": (d["vdim"],), p + "g": (hv, w), p + "o": (w, hv), p + "out": (w,)})
+        mlp = layer.get("mlp")
+        if not mlp:
+            continue
+        out[f"l{i}.norm2"] = (w,)
+        p = f"l{i}.mlp."
+        if mlp["kind"] == "dense":
+            out.update({p + "up": (mlp["ff"], w), p + "down": (w, mlp["ff"]), p + "act": (4,)})
+            continue
+        r, f = mlp["router"], mlp["expert"]["ff"]
+        total = r["experts"] + int(r.get("identity", 0) or 0)
+        out.update({p + "router": (total, w), p + "correction": (total,)})
+        for e in range(r["experts"]):
+            out.update({f"{p}e{e}.gate": (f, w), f"{p}e{e}.up": (f, w), f"{p}e{e}.down": (w, f)})
+        if mlp.get("shared"):
+            s = mlp["shared"]["ff"]
+            out.update({p + "shared.gate": (s, w), p + "shared.up": (s, w), p + "shared.down": (w, s), p + "shared.sg": (1, w)})
+    return out
+
+
+def random_weights(cfg: dict, seed: int) -> dict[str, torch.Tensor]:
+    """Random tensors whose values are exactly representable in bfloat16 (float64 here), drawn so that
+    every mechanism matters: projections of unit-size outputs (so that the experts' clamps bite), norm
+    weights near one, a router that prefers some experts clearly, corrections that change its choice
+    and make some choice scores negative, decays spread out."""
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, shape in tensor_shapes(cfg).items():
+        leaf = name.split(".")[-1]
+        if leaf in ("norm1", "norm2", "norm", "out"):
+            t = 1.0 + 0.2 * torch.randn(shape, generator=g)
+        elif leaf == "conv":
+            t = 0.6 * torch.randn(shape, generator=g)
+        elif leaf == "A_log":
+            t = torch.rand(shape, generator=g) * 2.0 - 1.5
+        elif leaf == "dt_bias":
+            t = torch.randn(shape, generator=g)
+        elif leaf == "act":
+            t = torch.tensor([1.0, 0.5, -0.3, 0.1]) + 0.2 * torch.randn(shape, generator=g)
+        elif leaf == "correction":
+            t = 0.15 * torch.randn(shape, generator=g) - 0.05
+        elif leaf == "router":
+            t = 3.0 * torch.randn(shape, generator=g) / math.sqrt(shape[-1])
+        elif name == "embed":
+            t = 0.5 * torch.randn(shape, generator=g)
+        else:
+            t = torch.randn(shape, generator=g) / math.sqrt(shape[-1]) * (2.0 if leaf in ("q", "k") else 1.0)
+        out[name] = t.to(torch.bfloat16).to(F)
+    return out
+
+
+def jittered(tensors: dict, seed: int = 0, size: float = 2.0 ** -8) -> dict:
+    """Every matrix with relative noise of the size of bfloat16's rounding: how far the logits of a
+    position move under it says how far rounding may move them."""
+    g = torch.Generator().manual_seed(seed)
+    return {n: t * (1 + size * torch.randn(t.shape, generator=g, dtype=F)) if t.dim() == 2 and not n.endswith("router") else t
+            for n, t in tensors.items()}
+
+
+def write_folder(folder, cfg: dict, tensors: dict):
+    """``config.json`` and ``model.safetensors`` (bfloat16) of ``tensors``, written byte by byte here."""
+    import json
+
+    import numpy as np
+
+    folder.mkdir(parents=True, exist_ok=True)
+    (folder / "config.json").write_text(json.dumps(cfg))
+    header, blobs, at = {}, [], 0
+    for name in sorted(tensors):
+        bits = (tensors[name].to(torch.float32).contiguous().view(torch.int32).numpy().astype(np.uint32) >> 16).astype("<u2")
+        raw = bits.tobytes()
+        header[name] = {"dtype": "BF16", "shape": list(tensors[name].shape), "data_offsets": [at, at + len(raw)]}
+        blobs.append(raw)
+        at += len(raw)
+    head = json.dumps(header).encode()
+    head += b" " * (-len(head) % 8)
+    with open(folder / "model.safetensors", "wb") as f:
+        f.write(len(head).to_bytes(8, "little") + head + b"".join(blobs))
+    return folder
