@@ -257,6 +257,24 @@ def makodra_shape(width, heads, kv_heads, ff, layers, vocab, chunk):
             "layers": [layer(order[i % 4]) for i in range(layers)]}
 
 
+def miberax_shape(width, heads, kv_heads, ff, layers, vocab, chunk):
+    """A Miberax of sizes that resemble a real model's layers: heads of 64 on both sides of every layer's
+    pair of mixers (the attention under a chunked mask with full rotation, the delta rule with as many
+    q/k heads as the attention has kv heads and a convolution of four taps), the feed-forward in turn
+    dense (the polynomial activation, the Llama layer's hidden size) and a mixture of 32 experts of an
+    eighth of that size, four of them chosen in four of eight groups, beside a shared expert of a quarter."""
+    def layer(i):
+        mixer = {"left": {"heads": heads, "kv_heads": kv_heads, "dim": 64, "vdim": 64, "scale": 0.125, "mask": {"size": chunk},
+                          "rot": {"dims": 64, "base": 1e6, "scaling": {"factor": 2.0}}},
+                 "right": {"heads": heads, "kv_heads": kv_heads, "dim": 64, "vdim": 64, "conv": 4}}
+        mlp = {"kind": "dense", "ff": ff} if i % 2 == 0 else {
+            "kind": "moe", "expert": {"ff": ff // 8, "limit": 7.0}, "shared": {"ff": ff // 4, "limit": 7.0},
+            "router": {"experts": 32, "top": 4, "identity": 0, "scale": 1.0, "groups": {"count": 8, "keep": 4}}}
+        return {"type": "parallel", "mixer": mixer, "mlp": mlp}
+    return {"architecture": "Miberax", "vocab": vocab, "width": width, "norm": {"eps": 1e-6, "groups": 4},
+            "layers": [layer(i) for i in range(layers)]}
+
+
 DESIGN_SIZES = {  # width, heads (of 64), kv heads, feed-forward, layers, vocabulary, attention chunk
     "1024": (1024, 16, 4, 4096, 8, 32000, 1024),
     "2048": (2048, 32, 8, 8192, 8, 32000, 2048),
@@ -274,6 +292,7 @@ def design_compare(args):
     for name in args.design_sizes.split(","):
         width, heads, kv_heads, ff, layers, vocab, chunk = DESIGN_SIZES[name]
         shapes = {
+            **({"miberax": miberax_shape(width, heads, kv_heads, ff, layers, vocab, chunk)} if args.design == "miberax" else {}),
             "makodra": makodra_shape(width, heads, kv_heads, ff, layers, vocab, chunk),
             "llama": dict(LLAMA_3_2_1B, vocab_size=vocab, hidden_size=width, intermediate_size=ff, num_hidden_layers=layers,
                           num_attention_heads=heads, num_key_value_heads=kv_heads, head_dim=64),
@@ -389,13 +408,13 @@ def main() -> int:
                     help="prompt length of --only-prefill (the line of the default run always has 2,048)")
     ap.add_argument("--portion", type=int, default=None,
                     help="with --only-prefill: the prompt runs in steps of at most this many tokens")
-    ap.add_argument("--design", default=None, choices=["makodra"],
+    ap.add_argument("--design", default=None, choices=["makodra", "miberax"],
                     help="instead of the default run: prefill (2,048 and 8,192 tokens) and decode (batch 1, 8, 64 at "
                          "--context) of this design beside the Llama decoder at equal sizes, random weights")
     ap.add_argument("--design-sizes", default="1024,2048", help="widths of --design, of " + ", ".join(DESIGN_SIZES))
     ap.add_argument("--design-phases", default="prefill2048,prefill8192,decode_b1,decode_b8,decode_b64",
                     help="with --design: which of these measurements to make")
-    ap.add_argument("--design-only", default=None, choices=["makodra", "llama"],
+    ap.add_argument("--design-only", default=None, choices=["makodra", "miberax", "llama"],
                     help="with --design: measure this one of the pair alone (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -419,7 +438,7 @@ def main() -> int:
     itemsize = 2 if short == "bf16" else 4
     if args.design:
         print(json.dumps({
-            "metric": f"{args.design} beside llama at equal sizes: prefill and decode tok/s", "unit": "tok/s", "n_gpus": 1,
+            "metric": f"{args.design} beside {'makodra and ' if args.design == 'miberax' else ''}llama at equal sizes: prefill and decode tok/s", "unit": "tok/s", "n_gpus": 1,
             "dtype": short, "data": "synthetic: random token ids, random-init weights N(0, 0.02)",
             "config": {"context": args.context, "kv_block_size": args.block_size, "sizes": {
                 n: dict(zip(("width", "heads_of_64", "kv_heads", "ff", "layers", "vocab", "chunk"), DESIGN_SIZES[n]))

@@ -50,44 +50,56 @@ struct PrepArgs {
   int entries, heads, kv_heads, dim, vdim, taps;
 };
 
-__global__ __launch_bounds__(256) void conv_prepare_kernel(PrepArgs p) {
-  extern __shared__ float y[];                                  // [channels]
-  const int row = blockIdx.x;
-  const int qk = p.kv_heads * p.dim, channels = 2 * qk + p.heads * p.vdim;
-  const int e = gd_entry_of_row(p.q_start, p.entries, row);
-  const int first = p.q_start[e];
-  const int pos = p.positions[row];
-  const float* kept = p.kept + (int64_t)p.state_slots[e] * p.state_stride;
-  for (int c = threadIdx.x; c < channels; c += blockDim.x) {
-    float acc = 0.f;
-    for (int j = p.taps - 1; j >= 0; --j) {                     // oldest input first
-      if (pos - j < 0) continue;                                // before the sequence: zero
-      const int src = row - j;
-      const float x = src >= first ? p.proj[(int64_t)src * p.stride + c]
-                                   : kept[(int64_t)(p.taps - 1 - (first - src)) * channels + c];
-      acc = fmaf(p.conv_w[(int64_t)c * p.taps + (p.taps - 1 - j)], x, acc);
-    }
-    y[c] = acc / (1.f + expf(-acc));
-  }
-  __syncthreads();
+// One input of the convolution of channel c, `back` places before `row` (which lies at position pos of
+// its request, whose step starts at row `first`): from the step's rows, from the kept inputs, or zero.
+__device__ __forceinline__ float conv_input(const PrepArgs& p, const float* kept, int channels, int row, int first, int pos,
+                                            int back, int c) {
+  if (pos - back < 0) return 0.f;                               // before the sequence
+  const int src = row - back;
+  return src >= first ? p.proj[(int64_t)src * p.stride + c] : kept[(int64_t)(p.taps - 1 - (first - src)) * channels + c];
+}
+
+__device__ __forceinline__ float conv_silu(const PrepArgs& p, const float* kept, int channels, int row, int first, int pos, int c) {
+  float acc = 0.f;
+  for (int j = p.taps - 1; j >= 0; --j)                         // oldest input first
+    acc = fmaf(p.conv_w[(int64_t)c * p.taps + (p.taps - 1 - j)], conv_input(p, kept, channels, row, first, pos, j, c), acc);
+  return acc / (1.f + expf(-acc));
+}
+
+// A wave a (row, unit). Units: the 2 kv_heads heads of q and k (convolution, silu, unit length), then the
+// channels of v in runs of 64 (convolution, silu), then one for beta and g of all heads.
+__global__ __launch_bounds__(64) void conv_prepare_kernel(PrepArgs p) {
+  const int row = blockIdx.x, unit = blockIdx.y, lane = threadIdx.x;
+  const int qk = p.kv_heads * p.dim, hv = p.heads * p.vdim, channels = 2 * qk + hv;
+  const int v_units = (hv + 63) / 64;
   float* out = p.out + (int64_t)row * p.out_stride;
-  const int lane = threadIdx.x % DLI_WAVE, wave = threadIdx.x / DLI_WAVE, waves = blockDim.x / DLI_WAVE;
-  const float q_scale = 1.f / sqrtf((float)p.dim);
-  for (int h = wave; h < 2 * p.kv_heads; h += waves) {          // q heads, then k heads
-    const float* src = y + (int64_t)h * p.dim;
-    float ss = 0.f;
-    for (int c = lane; c < p.dim; c += DLI_WAVE) ss += src[c] * src[c];
-    const float r = (1.f / sqrtf(wave_sum(ss) + 1e-6f)) * (h < p.kv_heads ? q_scale : 1.f);
-    for (int c = lane; c < p.dim; c += DLI_WAVE) out[(int64_t)h * p.dim + c] = src[c] * r;
+  if (unit == 2 * p.kv_heads + v_units) {
+    for (int h = lane; h < p.heads; h += DLI_WAVE) {
+      const float b = p.proj[(int64_t)row * p.stride + p.b_off + h];
+      const float a = p.proj[(int64_t)row * p.stride + p.a_off + h] + p.dt_bias[h];
+      const float softplus = a > 20.f ? a : log1pf(expf(a));
+      out[channels + h] = 1.f / (1.f + expf(-b));
+      out[channels + p.heads + h] = expf(-expf(p.a_log[h]) * softplus);
+    }
+    return;
   }
-  for (int c = 2 * qk + threadIdx.x; c < channels; c += blockDim.x) out[c] = y[c];
-  for (int h = threadIdx.x; h < p.heads; h += blockDim.x) {
-    const float b = p.proj[(int64_t)row * p.stride + p.b_off + h];
-    const float a = p.proj[(int64_t)row * p.stride + p.a_off + h] + p.dt_bias[h];
-    const float softplus = a > 20.f ? a : log1pf(expf(a));
-    out[channels + h] = 1.f / (1.f + expf(-b));
-    out[channels + p.heads + h] = expf(-expf(p.a_log[h]) * softplus);
+  const int e = gd_entry_of_row(p.q_start, p.entries, row);
+  const int first = p.q_start[e], pos = p.positions[row];
+  const float* kept = p.kept + (int64_t)p.state_slots[e] * p.state_stride;
+  if (unit >= 2 * p.kv_heads) {
+    const int c = 2 * qk + (unit - 2 * p.kv_heads) * 64 + lane;
+    if (c < channels) out[c] = conv_silu(p, kept, channels, row, first, pos, c);
+    return;
   }
+  const int c0 = unit * p.dim;                                  // q heads, then k heads
+  float ss = 0.f;
+  for (int c = lane; c < p.dim; c += DLI_WAVE) {
+    const float y = conv_silu(p, kept, channels, row, first, pos, c0 + c);
+    out[c0 + c] = y;
+    ss += y * y;
+  }
+  const float r = (1.f / sqrtf(wave_sum(ss) + 1e-6f)) * (unit < p.kv_heads ? 1.f / sqrtf((float)p.dim) : 1.f);
+  for (int c = lane; c < p.dim; c += DLI_WAVE) out[c0 + c] *= r;   // (each lane scales what it wrote itself)
 }
 
 // A thread a channel: it reads what it needs of the old kept inputs before it writes the new ones,
@@ -272,7 +284,7 @@ int dli_conv_prepare(const float* proj, int64_t stride, int b_off, int a_off, co
   if (rows <= 0 || entries <= 0) return DLI_OK;
   const int64_t channels = 2 * (int64_t)kv_heads * dim + (int64_t)heads * vdim;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0 || taps < 1 || taps > GD_MAX_TAPS ||
-      channels > 12288 || stride < channels || out_stride < channels + 2 * heads || b_off < channels || a_off < channels ||
+      stride < channels || out_stride < channels + 2 * heads || b_off < channels || a_off < channels ||
       b_off + heads > stride || a_off + heads > stride || state_stride < kept_offset + (taps - 1) * channels)
     return DLI_ERR_ARGUMENT;
   PrepArgs p;
@@ -280,7 +292,9 @@ int dli_conv_prepare(const float* proj, int64_t stride, int b_off, int a_off, co
   p.dt_bias = dt_bias; p.kept = state + kept_offset; p.state_stride = state_stride; p.q_start = q_start;
   p.positions = positions; p.state_slots = state_slots; p.out = out; p.out_stride = out_stride; p.entries = entries;
   p.heads = heads; p.kv_heads = kv_heads; p.dim = dim; p.vdim = vdim; p.taps = taps;
-  conv_prepare_kernel<<<rows, 256, channels * sizeof(float), stream>>>(p);
+  const int units = 2 * kv_heads + (int)(((int64_t)heads * vdim + 63) / 64) + 1;
+  if (units > 65535) return DLI_ERR_ARGUMENT;
+  conv_prepare_kernel<<<dim3(rows, units), 64, 0, stream>>>(p);
   if (dli_launch_status() != DLI_OK) return DLI_ERR_LAUNCH;
   if (taps > 1) {
     const dim3 grid(entries, (unsigned)((channels + 255) / 256));

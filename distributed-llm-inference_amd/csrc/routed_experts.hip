@@ -9,8 +9,9 @@
 //                    neighbours with the largest best choice stay; the `top` largest choices; weights = the chosen
 //                    scores (without correction) / (their sum + 1e-20) * scale
 //   expert_sort      the (token, choice) slots of real experts in runs by expert, and the list of row tiles
-//   expert_up/down   the experts' products over those tiles (vector units, any size), the clamped activation
-//                    between them; the down product leaves each slot's 32-bit result in the slot's own row
+//   expert_up/down   the experts' products over those tiles (on the matrix cores for bfloat16 and sizes that are
+//                    multiples of 32, else on the vector units, any size), the clamped activation between
+//                    them; the down product leaves each slot's 32-bit result in the slot's own row
 //   expert_combine   out = sum_j w_j (expert j's result, or the input itself for an identity expert)
 //                    + sigmoid(shared gate) * shared expert's result
 //
@@ -20,9 +21,10 @@
 
 __global__ void poly_norm_kernel_f32in(const float* __restrict__ z, int64_t z_stride, const float* __restrict__ coef,
                                        void* __restrict__ out_, int64_t out_stride, int ff, float eps, int out_is_bf16) {
-  __shared__ float scratch[16];
+  __shared__ float scratch[3][16];
   const int64_t row = blockIdx.x;
   const float* zr = z + row * z_stride;
+  const int lane = threadIdx.x % DLI_WAVE, wave = threadIdx.x / DLI_WAVE, waves = blockDim.x / DLI_WAVE;
   float s2 = 0.f, s4 = 0.f, s6 = 0.f;
   for (int i = threadIdx.x; i < ff; i += blockDim.x) {
     const float x = zr[i], x2 = x * x, x3 = x2 * x;
@@ -30,9 +32,13 @@ __global__ void poly_norm_kernel_f32in(const float* __restrict__ z, int64_t z_st
     s4 += x2 * x2;
     s6 += x3 * x3;
   }
-  const float r1 = 1.f / sqrtf(block_sum(s2, scratch) / (float)ff + eps);
-  const float r2 = 1.f / sqrtf(block_sum(s4, scratch) / (float)ff + eps);
-  const float r3 = 1.f / sqrtf(block_sum(s6, scratch) / (float)ff + eps);
+  // the three sums meet in one exchange through LDS
+  s2 = wave_sum(s2); s4 = wave_sum(s4); s6 = wave_sum(s6);
+  if (lane == 0) { scratch[0][wave] = s2; scratch[1][wave] = s4; scratch[2][wave] = s6; }
+  __syncthreads();
+  float t2 = 0.f, t4 = 0.f, t6 = 0.f;
+  for (int w = 0; w < waves; ++w) { t2 += scratch[0][w]; t4 += scratch[1][w]; t6 += scratch[2][w]; }   // same order in every thread
+  const float r1 = 1.f / sqrtf(t2 / (float)ff + eps), r2 = 1.f / sqrtf(t4 / (float)ff + eps), r3 = 1.f / sqrtf(t6 / (float)ff + eps);
   const float a = coef[0], b = coef[1], c = coef[2], e = coef[3];
   for (int i = threadIdx.x; i < ff; i += blockDim.x) {
     const float x = zr[i], x2 = x * x;
@@ -147,12 +153,13 @@ __global__ __launch_bounds__(64) void router_choose_kernel(const float* __restri
 #define EX_BK 16
 
 // One workgroup. ids [slots]: the chosen expert of every (token, choice) slot; ids at or above `experts`
-// (identity experts) have no rows. Leaves offsets [experts + 1], order [rows of real experts] (slot of
-// every sorted row), the tiles (expert, first sorted row) of at most EX_BM rows, and their number.
+// (identity experts) have no rows. Leaves offsets [experts + 1], order [rows of real experts] (the slot of
+// every sorted row; inside an expert's run the rows come in whatever order the counter hands out, which
+// no value depends on), the tiles (expert, first sorted row) of at most tile_rows rows, and their number.
 __global__ __launch_bounds__(1024) void expert_sort_kernel(const int* __restrict__ ids, int slots, int experts,
                                                            int* __restrict__ offsets, int* __restrict__ order,
                                                            int* __restrict__ tile_expert, int* __restrict__ tile_row0,
-                                                           int* __restrict__ tile_count, int max_tiles) {
+                                                           int* __restrict__ tile_count, int max_tiles, int tile_rows) {
   extern __shared__ int shi[];
   int *counts = shi, *cursor = shi + experts;
   for (int e = threadIdx.x; e < experts; e += blockDim.x) counts[e] = 0;
@@ -167,7 +174,7 @@ __global__ __launch_bounds__(1024) void expert_sort_kernel(const int* __restrict
     for (int e = 0; e < experts; ++e) {
       offsets[e] = at;
       cursor[e] = at;
-      for (int r = 0; r < counts[e] && tiles < max_tiles; r += EX_BM) {
+      for (int r = 0; r < counts[e] && tiles < max_tiles; r += tile_rows) {
         tile_expert[tiles] = e;
         tile_row0[tiles] = at + r;
         ++tiles;
@@ -178,22 +185,9 @@ __global__ __launch_bounds__(1024) void expert_sort_kernel(const int* __restrict
     tile_count[0] = tiles;
   }
   __syncthreads();
-  // Places inside an expert's run are handed out by an atomic counter; each run is then sorted by slot,
-  // so that the launch leaves the same lists from run to run (the values computed from them do not
-  // depend on the order either way).
   for (int i = threadIdx.x; i < slots; i += blockDim.x) {
     const int e = ids[i];
     if (e >= 0 && e < experts) order[atomicAdd(&cursor[e], 1)] = i;
-  }
-  __syncthreads();
-  for (int e = threadIdx.x; e < experts; e += blockDim.x) {
-    const int lo = offsets[e], hi = lo + counts[e];
-    for (int i = lo + 1; i < hi; ++i) {          // insertion sort: runs are short or nearly sorted
-      const int v = order[i];
-      int j = i - 1;
-      while (j >= lo && order[j] > v) { order[j + 1] = order[j]; --j; }
-      order[j + 1] = v;
-    }
   }
 }
 
@@ -304,6 +298,146 @@ __global__ __launch_bounds__(256) void expert_down_kernel(ExpertArgs p, const T*
   }
 }
 
+// The same two products on the matrix cores (bfloat16; width and ff multiples of 32): tiles of EXM_BM
+// sorted rows, a workgroup of four waves takes 128 features, each wave 32 of them (two blocks of 16) for
+// all rows of the tile. v_mfma_f32_16x16x32_bf16 with the weights as the first operand: lane l supplies
+// feature l % 16 of a block and row l % 16 of each block of 16 rows, and the eight k values
+// 8 (l / 16) .. + 7 of a step of 32, read straight from memory (16 bytes a lane and operand; the rows of
+// a tile are re-read by the four waves from the cache); the operands of the next step are asked for
+// before this step's products are issued. A lane's results are four neighbouring features of one row.
+// Every output sums its k in ascending steps of 32 whatever its tile, so a row's result depends on
+// nothing beside the row.
+#define EXM_BM 64
+#define EXM_MB (EXM_BM / 16)
+#define EXM_BN 128
+typedef __bf16 exm_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float exm_float4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ exm_bf16x8 exm_load(const bf16_t* p) { return *reinterpret_cast<const exm_bf16x8*>(p); }
+
+__global__ __launch_bounds__(256) void expert_up_mfma_kernel(ExpertArgs p, const bf16_t* __restrict__ h, int64_t h_stride,
+                                                             const bf16_t* __restrict__ w_gate,
+                                                             const bf16_t* __restrict__ w_up, bf16_t* __restrict__ y,
+                                                             float limit, float alpha) {
+  const int tile = blockIdx.x;
+  if (tile >= p.tile_count[0]) return;
+  const int e = p.tile_expert[tile], r0 = p.tile_row0[tile], rend = p.offsets[e + 1];
+  const int lane = threadIdx.x % DLI_WAVE, wave = threadIdx.x / DLI_WAVE;
+  const int c = lane % 16, kq = (lane / 16) * 8;
+  const int nw = blockIdx.y * EXM_BN + wave * 32;
+  const bf16_t *wg[2], *wu[2], *xr[EXM_MB];
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb) {
+    const int n = min(nw + nb * 16 + c, p.ff - 1);                              // (a feature past the end repeats the last)
+    wg[nb] = w_gate + ((int64_t)e * p.ff + n) * p.width + kq;
+    wu[nb] = w_up + ((int64_t)e * p.ff + n) * p.width + kq;
+  }
+#pragma unroll
+  for (int mb = 0; mb < EXM_MB; ++mb) {
+    const int r = min(r0 + mb * 16 + c, rend - 1);                              // (a row past the end repeats the last)
+    xr[mb] = h + (int64_t)(p.order[r] / p.top) * h_stride + kq;
+  }
+  exm_float4 accg[2][EXM_MB], accu[2][EXM_MB];
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+    for (int mb = 0; mb < EXM_MB; ++mb) accg[nb][mb] = accu[nb][mb] = exm_float4{0.f, 0.f, 0.f, 0.f};
+  const int blocks = (rend - r0 + 15) / 16;                                     // blocks of 16 rows that hold a row
+  exm_bf16x8 a[2], b[2], x[EXM_MB];
+  auto fetch = [&](int k) {
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) { a[nb] = exm_load(wg[nb] + k); b[nb] = exm_load(wu[nb] + k); }
+#pragma unroll
+    for (int mb = 0; mb < EXM_MB; ++mb) x[mb] = exm_load(xr[mb] + k);            // (unconditional: clamped rows are valid memory)
+  };
+  fetch(0);
+  for (int k = 0; k < p.width; k += 32) {
+    exm_bf16x8 a0[2], b0[2], x0[EXM_MB];
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) { a0[nb] = a[nb]; b0[nb] = b[nb]; }
+#pragma unroll
+    for (int mb = 0; mb < EXM_MB; ++mb) x0[mb] = x[mb];
+    fetch(min(k + 32, p.width - 32));                                           // the last turn asks for its own step again
+#pragma unroll
+    for (int mb = 0; mb < EXM_MB; ++mb) {
+      if (mb < blocks) {
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+          accg[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[nb], x0[mb], accg[nb][mb], 0, 0, 0);
+          accu[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b0[nb], x0[mb], accu[nb][mb], 0, 0, 0);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int mb = 0; mb < EXM_MB; ++mb) {
+    const int r = r0 + mb * 16 + c;
+    if (r >= rend) continue;
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+      const int n0 = nw + nb * 16 + (lane / 16) * 4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (n0 + i < p.ff) y[(int64_t)r * p.ff + n0 + i] = (bf16_t)clamped_glu(accg[nb][mb][i], accu[nb][mb][i], limit, alpha);
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void expert_down_mfma_kernel(ExpertArgs p, const bf16_t* __restrict__ y,
+                                                               const bf16_t* __restrict__ w_down, float* __restrict__ z) {
+  const int tile = blockIdx.x;
+  if (tile >= p.tile_count[0]) return;
+  const int e = p.tile_expert[tile], r0 = p.tile_row0[tile], rend = p.offsets[e + 1];
+  const int lane = threadIdx.x % DLI_WAVE, wave = threadIdx.x / DLI_WAVE;
+  const int c = lane % 16, kq = (lane / 16) * 8;
+  const int nw = blockIdx.y * EXM_BN + wave * 32;
+  const bf16_t *wd[2], *yr[EXM_MB];
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb) wd[nb] = w_down + ((int64_t)e * p.width + min(nw + nb * 16 + c, p.width - 1)) * p.ff + kq;
+#pragma unroll
+  for (int mb = 0; mb < EXM_MB; ++mb) yr[mb] = y + (int64_t)min(r0 + mb * 16 + c, rend - 1) * p.ff + kq;
+  exm_float4 acc[2][EXM_MB];
+#pragma unroll
+  for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+    for (int mb = 0; mb < EXM_MB; ++mb) acc[nb][mb] = exm_float4{0.f, 0.f, 0.f, 0.f};
+  const int blocks = (rend - r0 + 15) / 16;
+  exm_bf16x8 a[2], x[EXM_MB];
+  auto fetch = [&](int k) {
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) a[nb] = exm_load(wd[nb] + k);
+#pragma unroll
+    for (int mb = 0; mb < EXM_MB; ++mb) x[mb] = exm_load(yr[mb] + k);
+  };
+  fetch(0);
+  for (int k = 0; k < p.ff; k += 32) {
+    exm_bf16x8 a0[2], x0[EXM_MB];
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) a0[nb] = a[nb];
+#pragma unroll
+    for (int mb = 0; mb < EXM_MB; ++mb) x0[mb] = x[mb];
+    fetch(min(k + 32, p.ff - 32));
+#pragma unroll
+    for (int mb = 0; mb < EXM_MB; ++mb)
+      if (mb < blocks)
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) acc[nb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[nb], x0[mb], acc[nb][mb], 0, 0, 0);
+  }
+#pragma unroll
+  for (int mb = 0; mb < EXM_MB; ++mb) {
+    const int r = r0 + mb * 16 + c;
+    if (r >= rend) continue;
+    const int64_t slot = p.order[r];
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+      const int n0 = nw + nb * 16 + (lane / 16) * 4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (n0 + i < p.width) z[slot * p.width + n0 + i] = acc[nb][mb][i];
+    }
+  }
+}
+
 // out[token] = sum_j weights[token][j] * (ids[token][j] < experts ? z[token * top + j] : h[token])
 //            + sigmoid(shared_gate[token]) * shared[token]       (the shared expert, if there is one)
 template <typename T>
@@ -359,7 +493,9 @@ int dli_router_choose(const float* logits, int64_t stride, const float* correcti
   return dli_launch_status();
 }
 
-int dli_expert_tile_rows() { return EX_BM; }
+// Whether the matrix-core kernels take these sizes, and the rows of a tile of the kernels that will run.
+static bool expert_mfma(int width, int ff, int is_bf16) { return is_bf16 && width % 32 == 0 && ff % 32 == 0; }
+int dli_expert_tile_rows(int width, int ff, int is_bf16) { return expert_mfma(width, ff, is_bf16) ? EXM_BM : EX_BM; }
 
 // The experts' part of a mixture for `rows` tokens: sort, up product with activation, down product.
 // ids [rows][top]; scratch: offsets [experts + 1], order [rows * top], tile_expert and tile_row0 [max_tiles],
@@ -373,14 +509,23 @@ int dli_expert_products(const int* ids, const void* h, int64_t h_stride, const v
   if (top < 1 || experts < 1 || experts > 4096 || width <= 0 || ff <= 0 || h_stride < width || slots > (1 << 30) ||
       max_tiles < 1 || max_tiles > 65535 * 16)
     return DLI_ERR_ARGUMENT;
+  const bool mfma = expert_mfma(width, ff, is_bf16);
+  if (mfma && ((h_stride % 8) || ((uintptr_t)h % 16) || ((uintptr_t)w_gate % 16) || ((uintptr_t)w_up % 16) ||
+               ((uintptr_t)w_down % 16) || ((uintptr_t)y % 16)))
+    return DLI_ERR_ARGUMENT;
   expert_sort_kernel<<<1, 1024, 2 * experts * sizeof(int), stream>>>(ids, (int)slots, experts, offsets, order, tile_expert,
-                                                                     tile_row0, tile_count, max_tiles);
+                                                                     tile_row0, tile_count, max_tiles, mfma ? EXM_BM : EX_BM);
   if (dli_launch_status() != DLI_OK) return DLI_ERR_LAUNCH;
   ExpertArgs p;
   p.tile_expert = tile_expert; p.tile_row0 = tile_row0; p.tile_count = tile_count; p.offsets = offsets; p.order = order;
   p.top = top; p.width = width; p.ff = ff;
-  const dim3 up_grid(max_tiles, (ff + EX_BN - 1) / EX_BN), down_grid(max_tiles, (width + EX_BN - 1) / EX_BN);
-  if (is_bf16) {
+  const int bn = mfma ? EXM_BN : EX_BN;
+  const dim3 up_grid(max_tiles, (ff + bn - 1) / bn), down_grid(max_tiles, (width + bn - 1) / bn);
+  if (mfma) {
+    expert_up_mfma_kernel<<<up_grid, 256, 0, stream>>>(p, (const bf16_t*)h, h_stride, (const bf16_t*)w_gate,
+                                                       (const bf16_t*)w_up, (bf16_t*)y, limit, alpha);
+    expert_down_mfma_kernel<<<down_grid, 256, 0, stream>>>(p, (const bf16_t*)y, (const bf16_t*)w_down, z);
+  } else if (is_bf16) {
     expert_up_kernel<bf16_t><<<up_grid, 256, 0, stream>>>(p, (const bf16_t*)h, h_stride, (const bf16_t*)w_gate,
                                                           (const bf16_t*)w_up, (bf16_t*)y, limit, alpha);
     expert_down_kernel<bf16_t><<<down_grid, 256, 0, stream>>>(p, (const bf16_t*)y, (const bf16_t*)w_down, z);

@@ -262,29 +262,27 @@ __global__ void rotary_cache_kernel(const float* __restrict__ proj, int64_t stri
 }
 
 // x [rows][width] float32 (with delta: x += delta first, stored); each of `groups` equal consecutive
-// parts of the row is divided by its own root mean square; out(T) = w * that.
+// parts of the row is divided by its own root mean square; out(T) = w * that. A workgroup a (row, part).
 template <typename T>
 __global__ void group_norm_kernel(float* __restrict__ x, const float* __restrict__ delta, int64_t delta_stride,
                                   const float* __restrict__ weight, T* __restrict__ out, int width, int groups, float eps) {
   __shared__ float scratch[16];
   const int64_t row = blockIdx.x;
+  const int part = width / groups, first = blockIdx.y * part;
   float* xr = x + row * width;
-  const int part = width / groups;
-  for (int g = 0; g < groups; ++g) {
-    float ss = 0.f;
-    for (int i = g * part + threadIdx.x; i < (g + 1) * part; i += blockDim.x) {
-      float f = xr[i];
-      if (delta != nullptr) {
-        f += delta[row * delta_stride + i];
-        xr[i] = f;
-      }
-      ss += f * f;
+  float ss = 0.f;
+  for (int i = first + threadIdx.x; i < first + part; i += blockDim.x) {
+    float f = xr[i];
+    if (delta != nullptr) {
+      f += delta[row * delta_stride + i];
+      xr[i] = f;
     }
-    const float r = 1.f / sqrtf(block_sum(ss, scratch) / (float)part + eps);
-    // (each thread reads back what it wrote itself)
-    for (int i = g * part + threadIdx.x; i < (g + 1) * part; i += blockDim.x)
-      out[row * width + i] = from_f32<T>(weight[i] * (xr[i] * r));
+    ss += f * f;
   }
+  const float r = 1.f / sqrtf(block_sum(ss, scratch) / (float)part + eps);
+  // (each thread reads back what it wrote itself)
+  for (int i = first + threadIdx.x; i < first + part; i += blockDim.x)
+    out[row * width + i] = from_f32<T>(weight[i] * (xr[i] * r));
 }
 
 struct BranchArgs {
@@ -292,20 +290,40 @@ struct BranchArgs {
   int count;
 };
 
+// (the branches' sums of squares are made side by side and meet in one exchange through LDS; COUNT is a
+// template parameter so that no load hangs on a condition)
+template <int COUNT>
 __global__ void branch_norm_mean_kernel(BranchArgs b, float* __restrict__ out, int width, float eps) {
-  __shared__ float scratch[16];
+  __shared__ float scratch[COUNT][16];
   const int64_t row = blockIdx.x;
-  float r[4];
-  for (int j = 0; j < b.count; ++j) {
-    const float* yr = b.y[j] + row * b.stride[j];
-    float ss = 0.f;
-    for (int i = threadIdx.x; i < width; i += blockDim.x) ss += yr[i] * yr[i];
-    r[j] = 1.f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+  const int lane = threadIdx.x % DLI_WAVE, wave = threadIdx.x / DLI_WAVE, waves = blockDim.x / DLI_WAVE;
+  float ss[COUNT];
+#pragma unroll
+  for (int j = 0; j < COUNT; ++j) ss[j] = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x)
+#pragma unroll
+    for (int j = 0; j < COUNT; ++j) {
+      const float f = b.y[j][row * b.stride[j] + i];
+      ss[j] += f * f;
+    }
+#pragma unroll
+  for (int j = 0; j < COUNT; ++j) {
+    ss[j] = wave_sum(ss[j]);
+    if (lane == 0) scratch[j][wave] = ss[j];
   }
-  const float share = 1.f / (float)b.count;
+  __syncthreads();
+  float r[COUNT];
+#pragma unroll
+  for (int j = 0; j < COUNT; ++j) {
+    float total = 0.f;
+    for (int w = 0; w < waves; ++w) total += scratch[j][w];   // same order in every thread
+    r[j] = 1.f / sqrtf(total / (float)width + eps);
+  }
+  const float share = 1.f / (float)COUNT;
   for (int i = threadIdx.x; i < width; i += blockDim.x) {
     float sum = 0.f;
-    for (int j = 0; j < b.count; ++j) sum += b.weight[j][i] * (b.y[j][row * b.stride[j] + i] * r[j]);
+#pragma unroll
+    for (int j = 0; j < COUNT; ++j) sum += b.weight[j][i] * (b.y[j][row * b.stride[j] + i] * r[j]);
     out[row * width + i] = sum * share;
   }
 }
@@ -439,11 +457,13 @@ int dli_group_norm(float* x, const float* delta, int64_t delta_stride, const flo
                    int groups, float eps, int is_bf16, hipStream_t stream) {
   if (rows <= 0) return DLI_OK;
   if (width <= 0 || groups <= 0 || width % groups || (delta != nullptr && delta_stride < width)) return DLI_ERR_ARGUMENT;
-  const int threads = width / groups >= 1024 ? 512 : 256;
+  if (groups > 65535) return DLI_ERR_ARGUMENT;
+  const int part = width / groups, threads = part >= 2048 ? 512 : part >= 512 ? 256 : part >= 128 ? 128 : 64;
+  const dim3 grid(rows, groups);
   if (is_bf16)
-    group_norm_kernel<bf16_t><<<rows, threads, 0, stream>>>(x, delta, delta_stride, weight, (bf16_t*)out, width, groups, eps);
+    group_norm_kernel<bf16_t><<<grid, threads, 0, stream>>>(x, delta, delta_stride, weight, (bf16_t*)out, width, groups, eps);
   else
-    group_norm_kernel<float><<<rows, threads, 0, stream>>>(x, delta, delta_stride, weight, (float*)out, width, groups, eps);
+    group_norm_kernel<float><<<grid, threads, 0, stream>>>(x, delta, delta_stride, weight, (float*)out, width, groups, eps);
   return dli_launch_status();
 }
 
@@ -458,7 +478,12 @@ int dli_branch_norm_mean(const float* const* y, const int64_t* strides, const fl
     if (y[s] == nullptr || weights[s] == nullptr || strides[s] < width) return DLI_ERR_ARGUMENT;
     b.y[j] = y[s]; b.stride[j] = strides[s]; b.weight[j] = weights[s];
   }
-  branch_norm_mean_kernel<<<rows, 256, 0, stream>>>(b, out, width, eps);
+  switch (count) {
+    case 1: branch_norm_mean_kernel<1><<<rows, 256, 0, stream>>>(b, out, width, eps); break;
+    case 2: branch_norm_mean_kernel<2><<<rows, 256, 0, stream>>>(b, out, width, eps); break;
+    case 3: branch_norm_mean_kernel<3><<<rows, 256, 0, stream>>>(b, out, width, eps); break;
+    default: branch_norm_mean_kernel<4><<<rows, 256, 0, stream>>>(b, out, width, eps);
+  }
   return dli_launch_status();
 }
 

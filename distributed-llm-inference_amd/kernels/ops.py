@@ -133,7 +133,7 @@ _SIGNATURES = {
     "dli_poly_norm": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "dli_clamped_glu": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_float, _c_float, _c_int, _c_ptr],
     "dli_router_choose": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr, _c_ptr, _c_ptr],
-    "dli_expert_tile_rows": [],
+    "dli_expert_tile_rows": [_c_int, _c_int, _c_int],
     "dli_expert_products": [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
                             _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_int, _c_ptr],
     "dli_expert_combine": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int,
@@ -1887,7 +1887,7 @@ def expert_products(ids: torch.Tensor, h: torch.Tensor, w_gate: torch.Tensor, w_
     _require(w_up.shape == w_gate.shape and w_down.shape == (experts, width, ff) and h.shape == (n, width),
              "h [n, width], w_gate/w_up [experts, ff, width], w_down [experts, width, ff] do not fit")
     slots = n * top
-    tile_rows = int(library().dli_expert_tile_rows())
+    tile_rows = int(library().dli_expert_tile_rows(width, ff, _is_bf16(h.dtype)))
     max_tiles = max(1, min(slots, slots // tile_rows + experts))
     ints = torch.empty(experts + 1 + slots + 2 * max_tiles + 1, device=h.device, dtype=torch.int32)
     offsets, order = ints[:experts + 1], ints[experts + 1:experts + 1 + slots]

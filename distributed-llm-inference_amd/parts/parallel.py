@@ -5,7 +5,11 @@ one plus it), and the result is the mean of the branches.
 The branches are mixers of any kind, given as part specs with their own tensor prefixes; each keeps
 whatever it keeps per request (pages, a state, nothing), and the pair's cache is the composite of
 theirs. Norms, weights and the mean are 32-bit, and so is the result (it is a residual stream's
-next summand)."""
+next summand).
+
+Branches that begin with one product of their rows (``input_weight()`` answers with its matrix, and
+``forward`` takes the product's 32-bit result as ``proj``) share one product: their matrices are
+stacked at load and each gets its columns of the result."""
 
 from __future__ import annotations
 
@@ -15,6 +19,7 @@ import torch
 
 from ..kernels import ops
 from .base import CompositeCacheSpec, Mixer, Runtime
+from .linear import as_operand, linear_f32
 from .registry import build_part, register_part
 from .spec import PartSpec, WeightSpec
 
@@ -35,6 +40,8 @@ class ParallelMixers(Mixer):
         self.branches = {name: build_part("mixer", spec, runtime) for name, spec in branches.items()}
         self.out_names = {name: (out_weight_names or {}).get(name, f"{name}.out") for name in self.names}
         self.out_w: dict[str, torch.Tensor] = {}
+        self.w_in: Optional[torch.Tensor] = None      # the branches' first products as one
+        self.spans: dict[str, tuple[int, int]] = {}
 
     def sub_parts(self) -> dict:
         return dict(self.branches)
@@ -44,6 +51,18 @@ class ParallelMixers(Mixer):
 
     def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
         self.out_w = {n: tensors[self.out_names[n]].contiguous() for n in self.names if self.out_names[n] in tensors}
+
+    def finalize(self) -> None:
+        weights = {n: b.input_weight() if hasattr(b, "input_weight") else None for n, b in self.branches.items()}
+        if len(weights) < 2 or any(w is None for w in weights.values()):
+            return
+        at = 0
+        for n, w in weights.items():
+            self.spans[n] = (at, at + w.shape[0])
+            at += w.shape[0]
+        self.w_in = torch.cat(list(weights.values()), dim=0).contiguous()
+        for b in self.branches.values():
+            b.release_input_weight()
 
     def cache_spec(self) -> Optional[Any]:
         members = tuple((n, b.cache_spec()) for n, b in self.branches.items() if b.cache_spec() is not None)
@@ -57,8 +76,13 @@ class ParallelMixers(Mixer):
     def forward(self, x: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:
         members = cache.members if cache is not None and cache.kind == "composite" else {}
         outs = []
+        proj = linear_f32(self.rt, as_operand(self.rt, x, ctx), self.w_in) if self.w_in is not None else None
         for name in self.names:
-            y = self.branches[name].forward(x, ctx, members.get(name))
+            if proj is not None:
+                a, b = self.spans[name]
+                y = self.branches[name].forward(x, ctx, members.get(name), proj=proj[:, a:b])
+            else:
+                y = self.branches[name].forward(x, ctx, members.get(name))
             if y.dtype != torch.float32:
                 wide = torch.empty(y.shape, device=y.device, dtype=torch.float32)
                 ops.to_float(y, wide)

@@ -213,12 +213,21 @@ class GatedDelta(Mixer):
     def graph_capturable(self, page_size: int) -> bool:
         return True  # kernels on the context's device arrays only; padding rows write the spare slot
 
-    def forward(self, x: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:
+    def input_weight(self) -> Optional[torch.Tensor]:
+        """The matrix of the one product that reads the rows, for whoever stacks it with others'
+        (``forward`` then gets the product's result as ``proj``)."""
+        return self.w_in
+
+    def release_input_weight(self) -> None:
+        self.w_in = None
+
+    def forward(self, x: torch.Tensor, ctx: Any, cache: Any, proj: Optional[torch.Tensor] = None) -> torch.Tensor:
         if cache is None or cache.kind != "state" or not cache.writable:
             raise RuntimeError("gated_delta needs a state of its own")
         state = cache.state.view(cache.state.shape[0], -1)
         n, H = x.shape[0], self.num_heads
-        proj = linear_f32(self.rt, as_operand(self.rt, x, ctx), self.w_in)
+        if proj is None:
+            proj = linear_f32(self.rt, as_operand(self.rt, x, ctx), self.w_in)
         g_off = self.channels
         b_off, a_off = g_off + self.hv, g_off + self.hv + H
         prep = torch.empty(n, self.channels + 2 * H, device=self.rt.device, dtype=torch.float32)

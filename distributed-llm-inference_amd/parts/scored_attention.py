@@ -32,7 +32,7 @@ import torch
 
 from ..kernels import ops
 from .base import Mixer, PagedKVSpec, PositionEncoding, Runtime
-from .linear import as_operand, linear_f32
+from .linear import as_operand, linear_f32, stack_rows
 from .registry import build_part, register_part
 from .spec import PartSpec, WeightSpec
 
@@ -107,7 +107,7 @@ class ScoredAttention(Mixer):
     def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
         n = self.names
         stacked = [tensors[n["q"]], tensors[n["k"]], tensors[n["v"]]] + ([tensors[n["g"]]] if self.output_gate else [])
-        self.w_in = torch.cat(stacked, dim=0).contiguous()
+        self.w_in = stack_rows(stacked)
         self.w_o = tensors[n["o"]]
         if self.distance_penalty:
             self.r1, self.r2 = tensors[n["r1"]].contiguous(), tensors[n["r2"]].contiguous()
@@ -132,12 +132,21 @@ class ScoredAttention(Mixer):
     def graph_capturable(self, page_size: int) -> bool:
         return True  # a step of single tokens is read through the context's device arrays alone
 
-    def forward(self, x: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:
+    def input_weight(self) -> Optional[torch.Tensor]:
+        """The matrix of the one product that reads the rows, for whoever stacks it with others'
+        (``forward`` then gets the product's result as ``proj``)."""
+        return self.w_in
+
+    def release_input_weight(self) -> None:
+        self.w_in = None
+
+    def forward(self, x: torch.Tensor, ctx: Any, cache: Any, proj: Optional[torch.Tensor] = None) -> torch.Tensor:
         if cache is None or cache.kind != "paged" or not cache.writable:
             raise RuntimeError("scored_attention needs a paged cache of its own")
         grp = ctx.groups[cache.group]
         n = x.shape[0]
-        proj = linear_f32(self.rt, as_operand(self.rt, x, ctx), self.w_in)
+        if proj is None:
+            proj = linear_f32(self.rt, as_operand(self.rt, x, ctx), self.w_in)
         q = self.rt.empty(n, self._q)
         first_in = first_out = None
         if self.value_mix == "source":
@@ -157,7 +166,8 @@ class ScoredAttention(Mixer):
                              0 if table is None else table.dim, table is not None and table.pairing == "interleaved",
                              q, grp.slots, cache.k_pages, cache.v_pages, self.num_heads)
         out = self.rt.empty(n, self._o)
-        gate = proj[:, self._q + self._k + self._v:] if self.output_gate else None
+        g0 = self._q + self._k + self._v
+        gate = proj[:, g0:g0 + self._o] if self.output_gate else None
         changes = dict(window=self.window, chunk=self.chunk, sink=self.sink, r1=self.r1, r2=self.r2)
         nd = ctx.num_decode
         if nd == ctx.num_entries:
