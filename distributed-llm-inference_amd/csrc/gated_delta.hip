@@ -1,7 +1,7 @@
 // The gated delta rule: a matrix state S [key][value] per head in 32-bit, carried from token to token
 // of a request in its state slot, with one decay g and one write strength beta per head and token:
 //
-//   S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q      (the read-out sees the write)
+//   S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q      (in this order: o is made from the state that already holds the token)
 //
 // Keys and values may differ in size (D keys, V values a head), and several value heads may share
 // the q and k of one of `kv_heads` heads. Around it, in the same 32-bit arithmetic:

@@ -123,7 +123,7 @@ def test_composite_caches_in_the_store():
 def test_plain_mechanisms_agree_with_their_definitions():
     torch.manual_seed(0)
     F = torch.float64
-    # the recurrence's read-out sees the current token's write: one token, zero state
+    # o is made from the state that already holds the token: one token, zero state
     q, k, v = torch.randn(1, 1, 4, dtype=F), torch.randn(1, 1, 4, dtype=F), torch.randn(1, 1, 3, dtype=F)
     o = P.gated_delta_rule(q, k, v, torch.tensor([[0.5]], dtype=F), torch.tensor([[0.9]], dtype=F))
     assert torch.allclose(o[0, 0], 0.5 * v[0, 0] * (k[0, 0] @ q[0, 0]))
