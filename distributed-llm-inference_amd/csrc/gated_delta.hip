@@ -236,7 +236,7 @@ __global__ __launch_bounds__(64) void gated_delta_scan_kernel(GdArgs p) {
 // Any D and V: a thread a value column, the column's state in the request's slot.
 __global__ void gated_delta_any_kernel(GdArgs p, int D) {
   extern __shared__ float sh[];
-  float *sk = sh, *sq = sh + D, *scratch = sh + 2 * D;
+  float *sk = sh, *sq = sh + D;
   const int v = blockIdx.z * blockDim.x + threadIdx.x, V = p.vdim;
   const bool live = v < V;
   const int entry = blockIdx.x, head = blockIdx.y;
@@ -270,7 +270,6 @@ __global__ void gated_delta_any_kernel(GdArgs p, int D) {
     for (int c = 0; c < D; ++c) st[c] = fmaf(sk[c], u, g * st[c]);
     p.o[row * p.o_stride + (int64_t)head * V + v] = fmaf(u, kq, g * qs);
   }
-  (void)scratch;
 }
 
 extern "C" {
@@ -328,7 +327,7 @@ int dli_gated_delta_scan(const float* prep, int64_t stride, float* state, int64_
     GD_CASE(12, 4) GD_CASE(16, 4)
     default: {
       const int threads = vdim >= 256 ? 256 : (vdim + 63) / 64 * 64;
-      gated_delta_any_kernel<<<dim3(entries, heads, (vdim + threads - 1) / threads), threads, (2 * dim + 16) * sizeof(float),
+      gated_delta_any_kernel<<<dim3(entries, heads, (vdim + threads - 1) / threads), threads, 2 * dim * sizeof(float),
                                stream>>>(p, dim);
     }
   }

@@ -21,7 +21,7 @@ one kernel adds everything up in 32-bit. The expert matrices are stacked ``[expe
 
 from __future__ import annotations
 
-from typing import Any, Mapping, Optional
+from typing import Any, Mapping
 
 import torch
 
